@@ -1,0 +1,59 @@
+"""Compile the two shared libraries of the package, in-tree.
+
+    libmuxhost.so  - g++,   pure host C++ (allocator + batch builder)
+    libmuxattn.so  - hipcc, gfx950 kernels + their C ABI
+
+Run as ``python -m muxserve_amd.build``.  Nothing here runs at import time of
+the package: the loaders in muxserve_amd._lib only open what this step built
+and raise if it is missing.
+"""
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+INCLUDE = os.path.join(ROOT, "include")
+CSRC = os.path.join(PKG, "csrc")
+
+HOST_LIB = os.path.join(PKG, "libmuxhost.so")
+ATTN_LIB = os.path.join(PKG, "libmuxattn.so")
+
+HOST_SOURCES = [os.path.join(CSRC, "host", f) for f in ("kv_storage.cpp", "batch_scheduler.cpp")]
+HIP_SOURCES = [os.path.join(CSRC, "hip", f) for f in (
+    "cache_write.hip", "paged_decode.hip", "prefill.hip", "runtime.hip")]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# Packed-FP32 instruction selection is switched off for every device
+# translation unit (ordinary float code otherwise compiles to v_pk_*_f32).
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-fno-gpu-rdc", "-Wno-unused-command-line-argument"]
+
+
+def _run(cmd):
+    print("[build]", " ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build_host():
+    _run(["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-Wextra",
+          f"-I{INCLUDE}", *HOST_SOURCES, "-o", HOST_LIB])
+    return HOST_LIB
+
+
+def build_hip(extra=()):
+    srcs = [s for s in HIP_SOURCES if os.path.exists(s)]
+    _run([HIPCC, *HIP_FLAGS, *extra, f"-I{INCLUDE}", f"-I{os.path.join(CSRC, 'hip')}",
+          *srcs, "-o", ATTN_LIB])
+    return ATTN_LIB
+
+
+def build_all():
+    build_host()
+    build_hip()
+
+
+if __name__ == "__main__":
+    what = sys.argv[1] if len(sys.argv) > 1 else "all"
+    {"host": build_host, "hip": build_hip, "all": build_all}[what]()
