@@ -1,0 +1,162 @@
+/*
+ * muxserve_attn.h - C ABI of the device half of the hot path (libmuxattn.so,
+ * HIP, gfx950): KV-cache write, paged decode attention and causal prefill
+ * attention over the unified head-granular KV block pool, plus CU-masked
+ * stream creation for prefill/decode colocation.
+ *
+ * What these replace.  In the reference the attention layer is constructed at
+ * muxserve/flexserver/models/llama.py:138-147 and invoked at
+ * muxserve/flexserver/models/llama.py:159-161 as
+ *     attn(positions, q, k, v, k_cache, v_cache, input_metadata, cache_event)
+ * with k_cache/v_cache the WHOLE pool (models/llama.py:276-288,
+ * pipeworker.py:93-106) and the index tensors built at
+ * muxserve/flexserver/llm_runtime.py:300-334.  The arithmetic behind that call
+ * lives in the external MuxServe-vLLM fork (cache_ops.reshape_and_cache,
+ * attention_ops.paged_attention, the prefill attention); the entry points
+ * below are what a binding for that call would link instead.
+ *
+ * Pool layout (muxserve/flexstore/manager.py:456-468, 485-492), one entry per
+ * (token block, layer, head) - "head-block":
+ *     K pool  [num_blocks, D/x, block_size, x]   x = 16 / sizeof(elem) = 8
+ *     V pool  [num_blocks, D,   block_size]
+ * D (head size) is 128 (manager.py:337).  A slot is block_id*block_size+offset
+ * (csrc/batch_scheduler.h:50-53).
+ *
+ * Conventions: every pointer is a DEVICE pointer owned by the caller unless
+ * noted; nothing is retained past the call; all work is enqueued on `stream`
+ * (a hipStream_t passed as void*; NULL = the default stream) and the call
+ * returns without synchronising.  Return value: 0 on success, a negative
+ * MUXA_E* code on a rejected argument; no exceptions cross the boundary.
+ * Shapes are validated on the host before any launch.
+ */
+#ifndef MUXSERVE_ATTN_H
+#define MUXSERVE_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MUXA_OK 0
+#define MUXA_EINVAL (-1)      /* null pointer / negative size / bad stride     */
+#define MUXA_EUNSUPPORTED (-2)/* head size != 128, block size not 8/16/32 ...  */
+#define MUXA_EWORKSPACE (-3)  /* workspace missing or too small                */
+#define MUXA_EHIP (-4)        /* a HIP runtime call failed (see mux_last_hip_error) */
+
+#define MUXA_DTYPE_F16 0
+#define MUXA_DTYPE_BF16 1
+
+#define MUXA_MAX_DECODE_ITEMS 8
+
+/* Library version (major*10000 + minor*100 + patch). */
+int32_t mux_attn_version(void);
+/* hipError_t of the last failing HIP call made by this library on the calling
+ * thread (0 if none). */
+int32_t mux_last_hip_error(void);
+
+/* ---- KV-cache write ------------------------------------------------------
+ * Stands in for cache_ops.reshape_and_cache as called by the attention layer
+ * behind models/llama.py:159-161: for token t, kv-head h, dim d
+ *     slot = slot_mapping[t, layer, h]; b = slot / block_size; o = slot % block_size
+ *     K_pool[b, d/8, o, d%8] = k[t, h, d];   V_pool[b, d, o] = v[t, h, d]
+ * k, v: [num_tokens, Hkv*D] with row stride kv_row_stride (elements; q,k,v are
+ * column slices of one qkv row, models/llama.py:157-158).  slot_mapping: int64
+ * [num_tokens, L, Hkv] as built at llm_runtime.py:301-302.  Slots < 0 are
+ * skipped.  Bit-exact byte movement; no arithmetic. */
+int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t kv_row_stride,
+                              void *k_pool, void *v_pool, int64_t num_pool_blocks,
+                              const int64_t *slot_mapping, int32_t layer, int32_t num_layers,
+                              int32_t num_tokens, int32_t num_kv_heads, int32_t head_size,
+                              int32_t block_size, int32_t dtype, void *stream);
+
+/* ---- Paged decode attention ---------------------------------------------
+ * One model's decode step for one layer; stands in for
+ * attention_ops.paged_attention behind models/llama.py:159-161.  For sequence
+ * s and query head hq (kv head hk = hq / (Hq/Hkv)):
+ *     out[s,hq,:] = softmax(scale * q[s,hq,:] . K[0:ctx_s]) . V[0:ctx_s]
+ * with K/V gathered block by block through block_tables[layer, s, hk, :].
+ * fp16/bf16 storage, fp32 accumulation.
+ *
+ * q, out: [>=num_seqs, Hq*D], row strides in elements.
+ * block_tables: int32 [L, num_seqs, Hkv, max_blocks] (llm_runtime.py:327);
+ * only the first ceil(ctx/block_size) entries of a row are read.
+ * context_lens: int32 [num_seqs].  max_context_len: host-side upper bound on
+ * context_lens (InputMetadata.max_context_len, pipeworker.py:81-90); it sizes
+ * the grid, device values above it are clamped.
+ * partition_size: tokens per split of a context (multiple of 64), 0 = choose.
+ * workspace: scratch for split partials, at least
+ * mux_paged_decode_workspace_bytes(...) bytes; may be NULL when that is 0. */
+typedef struct MuxDecodeItem {
+  void *out;
+  const void *q;
+  int64_t out_row_stride;
+  int64_t q_row_stride;
+  const int32_t *block_tables;   /* base of the [L, B, Hkv, max_blocks] tensor */
+  const int32_t *context_lens;
+  int32_t layer;
+  int32_t num_layers;
+  int32_t num_seqs;
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  int32_t max_blocks;
+  int32_t max_context_len;
+  float scale;
+} MuxDecodeItem;
+
+size_t mux_paged_decode_workspace_bytes(const MuxDecodeItem *items, int32_t n_items,
+                                        int32_t partition_size);
+
+/* Fused launch over up to MUXA_MAX_DECODE_ITEMS models that share the pool,
+ * head size, block size and dtype ("mixed multi-LLM decode": one grid covers
+ * every model's (sequence, head, partition) work).  `items` is a HOST array. */
+int32_t mux_multi_decode(const MuxDecodeItem *items, int32_t n_items,
+                         const void *k_pool, const void *v_pool, int64_t num_pool_blocks,
+                         int32_t head_size, int32_t block_size, int32_t dtype,
+                         int32_t partition_size, void *workspace, size_t workspace_bytes,
+                         void *stream);
+
+/* Single-model convenience wrapper around mux_multi_decode. */
+int32_t mux_paged_decode(void *out, int64_t out_row_stride, const void *q, int64_t q_row_stride,
+                         const void *k_pool, const void *v_pool, int64_t num_pool_blocks,
+                         const int32_t *block_tables, const int32_t *context_lens,
+                         int32_t layer, int32_t num_layers, int32_t num_seqs,
+                         int32_t num_q_heads, int32_t num_kv_heads, int32_t head_size,
+                         int32_t block_size, int32_t max_blocks, int32_t max_context_len,
+                         float scale, int32_t dtype, int32_t partition_size,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- Causal prefill attention -------------------------------------------
+ * Stands in for the prompt branch of the attention layer behind
+ * models/llama.py:159-161: per prompt p (tokens cu_seqlens[p]..cu_seqlens[p+1])
+ *     out[t,hq,:] = softmax(scale * q[t,hq,:] . k[<=t,hk,:]) . v[<=t,hk,:]
+ * on the fresh q,k,v (the pool is not read).  cu_seqlens: DEVICE int32
+ * [num_prompts+1] prefix sums of InputMetadata.prompt_lens; max_prompt_len is
+ * a host-side upper bound that sizes the grid. */
+int32_t mux_prefill_causal(void *out, int64_t out_row_stride,
+                           const void *q, int64_t q_row_stride,
+                           const void *k, const void *v, int64_t kv_row_stride,
+                           const int32_t *cu_seqlens, int32_t num_prompts, int32_t max_prompt_len,
+                           int32_t num_q_heads, int32_t num_kv_heads, int32_t head_size,
+                           float scale, int32_t dtype, void *stream);
+
+/* ---- CU-masked streams ---------------------------------------------------
+ * Replacement for the reference's per-process MPS share
+ * (CUDA_MPS_ACTIVE_THREAD_PERCENTAGE, muxserve/muxsched/launcher.py:54-61):
+ * a stream whose kernels run only on the compute units selected by bits
+ * [lo_percent*N/100, hi_percent*N/100) of the device's N-bit CU mask.  The
+ * kernel driver deals consecutive mask bits round-robin over XCDs and shader
+ * engines, so a contiguous bit range is a share spread evenly over the chip,
+ * and two disjoint ranges never share a CU.  *stream_out receives a
+ * hipStream_t; *num_cus_out (optional) the number of CUs enabled. */
+int32_t mux_stream_create_cu_range(void **stream_out, int32_t lo_percent, int32_t hi_percent,
+                                   int32_t *num_cus_out);
+int32_t mux_stream_destroy(void *stream);
+/* Device facts used by the mask builder: out = [num_cus, num_xcds]. */
+int32_t mux_device_cu_info(int32_t out[2]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MUXSERVE_ATTN_H */

@@ -84,3 +84,70 @@ def check_host(rc, what):
             raise MemoryError(msg)
         raise ValueError(msg)
     return rc
+
+
+# ---------------------------------------------------------------------------
+# libmuxattn.so (include/muxserve_attn.h)
+# ---------------------------------------------------------------------------
+c_f32 = ctypes.c_float
+c_sz = ctypes.c_size_t
+
+MUXA_MAX_DECODE_ITEMS = 8
+DTYPE_F16, DTYPE_BF16 = 0, 1
+
+
+class MuxDecodeItem(ctypes.Structure):
+    _fields_ = [
+        ("out", c_vp), ("q", c_vp),
+        ("out_row_stride", c_i64), ("q_row_stride", c_i64),
+        ("block_tables", c_vp), ("context_lens", c_vp),
+        ("layer", c_i32), ("num_layers", c_i32), ("num_seqs", c_i32),
+        ("num_q_heads", c_i32), ("num_kv_heads", c_i32),
+        ("max_blocks", c_i32), ("max_context_len", c_i32),
+        ("scale", c_f32),
+    ]
+
+
+ATTN_SIGNATURES = {
+    "mux_attn_version": (c_i32, []),
+    "mux_last_hip_error": (c_i32, []),
+    "mux_reshape_and_cache": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i32, c_i32,
+                                      c_i32, c_i32, c_i32, c_i32, c_i32, c_vp]),
+    "mux_paged_decode_workspace_bytes": (c_sz, [c_vp, c_i32, c_i32]),
+    "mux_multi_decode": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_i32,
+                                 c_vp, c_sz, c_vp]),
+    "mux_paged_decode": (c_i32, [c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_vp,
+                                 c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32,
+                                 c_f32, c_i32, c_i32, c_vp, c_sz, c_vp]),
+    "mux_prefill_causal": (c_i32, [c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i32, c_i32,
+                                   c_i32, c_i32, c_i32, c_f32, c_i32, c_vp]),
+    "mux_stream_create_cu_range": (c_i32, [c_vp, c_i32, c_i32, c_vp]),
+    "mux_stream_destroy": (c_i32, [c_vp]),
+    "mux_device_cu_info": (c_i32, [c_vp]),
+}
+
+
+def attn():
+    """libmuxattn.so with argument/return types declared."""
+    global _attn
+    if _attn is not None:
+        return _attn
+    lib = _open(ATTN_LIB_PATH)
+    for name, (res, args) in ATTN_SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _attn = lib
+    return lib
+
+
+ATTN_ERRORS = {-1: "invalid argument", -2: "unsupported shape or dtype",
+               -3: "workspace missing or too small", -4: "HIP runtime error"}
+
+
+def check_attn(rc, what):
+    if rc != 0:
+        extra = ""
+        if rc == -4:
+            extra = f", hipError {attn().mux_last_hip_error()}"
+        raise RuntimeError(f"{what}: {ATTN_ERRORS.get(int(rc), 'error')} (code {int(rc)}{extra})")

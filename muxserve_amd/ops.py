@@ -1,0 +1,185 @@
+"""Tensor-level wrappers over the C ABI of libmuxattn.so.
+
+torch is used here for device memory and streams only: every function takes
+CUDA(HIP) tensors, checks what the C ABI cannot (device, dtype, contiguity of
+the innermost dimension), and passes raw pointers plus the current stream.
+There is no fallback: without the library, or with CPU tensors, these raise.
+"""
+import ctypes
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+
+from . import _lib
+
+HEAD_SIZE = 128   # muxserve/flexstore/manager.py:337
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float16:
+        return _lib.DTYPE_F16
+    if t.dtype == torch.bfloat16:
+        return _lib.DTYPE_BF16
+    raise TypeError(f"expected float16 or bfloat16, got {t.dtype}")
+
+
+def _need_cuda(*tensors):
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("muxserve_amd.ops: tensors must live on the GPU (no CPU path)")
+
+
+def _stream_ptr(stream=None) -> int:
+    if stream is None:
+        return torch.cuda.current_stream().cuda_stream
+    if isinstance(stream, int):
+        return stream
+    return stream.cuda_stream
+
+
+def _rows(t: torch.Tensor, what: str) -> int:
+    """Row stride (elements) of a 2-D [rows, width] tensor with unit inner stride."""
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise ValueError(f"{what}: expected [rows, width] with contiguous rows")
+    return t.stride(0)
+
+
+def pool_block_size(k_pool: torch.Tensor) -> int:
+    """K pool is [N, D/8, block_size, 8] (muxserve/flexstore/manager.py:456-462)."""
+    if k_pool.dim() != 4 or k_pool.shape[1] * k_pool.shape[3] != HEAD_SIZE or k_pool.shape[3] != 8:
+        raise ValueError(f"k_pool: expected [N, 16, block_size, 8], got {tuple(k_pool.shape)}")
+    return int(k_pool.shape[2])
+
+
+def _check_pools(k_pool, v_pool):
+    bs = pool_block_size(k_pool)
+    if tuple(v_pool.shape) != (k_pool.shape[0], HEAD_SIZE, bs):
+        raise ValueError(f"v_pool: expected {(k_pool.shape[0], HEAD_SIZE, bs)}, got {tuple(v_pool.shape)}")
+    if not (k_pool.is_contiguous() and v_pool.is_contiguous()):
+        raise ValueError("pools must be contiguous")
+    if k_pool.dtype != v_pool.dtype:
+        raise TypeError("k_pool and v_pool dtypes differ")
+    return bs
+
+
+def reshape_and_cache(k: torch.Tensor, v: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                      slot_mapping: torch.Tensor, layer: int = 0, num_tokens: Optional[int] = None,
+                      stream=None) -> None:
+    """Scatter k, v [T_pad, Hkv*128] into the pool through slot_mapping
+    int64 [T, L, Hkv] (slice `layer`).  Rows >= T of k/v are padding
+    (muxserve/flexserver/llm_runtime.py:300) and are not read."""
+    _need_cuda(k, v, k_pool, v_pool, slot_mapping)
+    bs = _check_pools(k_pool, v_pool)
+    if slot_mapping.dtype != torch.int64 or slot_mapping.dim() != 3 or not slot_mapping.is_contiguous():
+        raise ValueError("slot_mapping: expected contiguous int64 [T, L, Hkv]")
+    T, L, H = slot_mapping.shape
+    if num_tokens is not None:
+        T = min(T, int(num_tokens))
+    stride = _rows(k, "k")
+    if _rows(v, "v") != stride or k.shape != v.shape or k.dtype != v.dtype or k.dtype != k_pool.dtype:
+        raise ValueError("k and v must have the same shape, strides and dtype as each other and the pool's dtype")
+    if k.shape[0] < T or k.shape[1] != H * HEAD_SIZE:
+        raise ValueError(f"k: expected [>={T}, {H * HEAD_SIZE}], got {tuple(k.shape)}")
+    rc = _lib.attn().mux_reshape_and_cache(
+        k.data_ptr(), v.data_ptr(), stride, k_pool.data_ptr(), v_pool.data_ptr(), k_pool.shape[0],
+        slot_mapping.data_ptr(), int(layer), L, T, H, HEAD_SIZE, bs, _dtype_code(k), _stream_ptr(stream))
+    _lib.check_attn(rc, "mux_reshape_and_cache")
+
+
+@dataclass
+class DecodeCall:
+    """One model's decode step for one layer (an element of a fused launch)."""
+    out: torch.Tensor             # [>=B, Hq*128]
+    q: torch.Tensor               # [>=B, Hq*128] (may be a column slice of qkv)
+    block_tables: torch.Tensor    # int32 [L, B, Hkv, max_blocks]
+    context_lens: torch.Tensor    # int32 [B]
+    max_context_len: int
+    scale: float
+    layer: int = 0
+
+    def to_item(self) -> _lib.MuxDecodeItem:
+        bt, cl = self.block_tables, self.context_lens
+        _need_cuda(self.out, self.q, bt, cl)
+        if bt.dtype != torch.int32 or bt.dim() != 4 or not bt.is_contiguous():
+            raise ValueError("block_tables: expected contiguous int32 [L, B, Hkv, max_blocks]")
+        if cl.dtype != torch.int32 or cl.dim() != 1 or not cl.is_contiguous():
+            raise ValueError("context_lens: expected contiguous int32 [B]")
+        L, B, Hkv, max_blocks = bt.shape
+        if cl.shape[0] != B:
+            raise ValueError("context_lens and block_tables disagree on the number of sequences")
+        if self.q.shape[1] % HEAD_SIZE or self.q.shape[0] < B or self.out.shape != self.q.shape:
+            raise ValueError("q/out: expected [>=B, Hq*128] of equal shape")
+        if self.q.dtype != self.out.dtype:
+            raise TypeError("q and out dtypes differ")
+        it = _lib.MuxDecodeItem()
+        it.out, it.q = self.out.data_ptr(), self.q.data_ptr()
+        it.out_row_stride, it.q_row_stride = _rows(self.out, "out"), _rows(self.q, "q")
+        it.block_tables, it.context_lens = bt.data_ptr(), cl.data_ptr()
+        it.layer, it.num_layers, it.num_seqs = int(self.layer), L, B
+        it.num_q_heads, it.num_kv_heads = self.q.shape[1] // HEAD_SIZE, Hkv
+        it.max_blocks, it.max_context_len = max_blocks, int(self.max_context_len)
+        it.scale = float(self.scale)
+        return it
+
+
+_workspaces = {}
+
+
+def _workspace(nbytes: int, device) -> Optional[torch.Tensor]:
+    """Grow-only scratch for split partials, one per (device, stream)."""
+    if nbytes == 0:
+        return None
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def multi_decode(calls: List[DecodeCall], k_pool: torch.Tensor, v_pool: torch.Tensor,
+                 partition_size: int = 0, workspace: Optional[torch.Tensor] = None, stream=None) -> None:
+    """Paged decode attention for several colocated models in one launch."""
+    if not 1 <= len(calls) <= _lib.MUXA_MAX_DECODE_ITEMS:
+        raise ValueError(f"1..{_lib.MUXA_MAX_DECODE_ITEMS} models per launch")
+    _need_cuda(k_pool, v_pool)
+    bs = _check_pools(k_pool, v_pool)
+    items = (_lib.MuxDecodeItem * len(calls))(*[c.to_item() for c in calls])
+    for c in calls:
+        if c.q.dtype != k_pool.dtype:
+            raise TypeError("q dtype must equal the pool dtype")
+    lib = _lib.attn()
+    need = lib.mux_paged_decode_workspace_bytes(ctypes.addressof(items), len(calls), int(partition_size))
+    ws = workspace if workspace is not None else _workspace(need, k_pool.device)
+    ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)
+    rc = lib.mux_multi_decode(ctypes.addressof(items), len(calls), k_pool.data_ptr(), v_pool.data_ptr(),
+                              k_pool.shape[0], HEAD_SIZE, bs, _dtype_code(k_pool), int(partition_size),
+                              ws_ptr, ws_bytes, _stream_ptr(stream))
+    _lib.check_attn(rc, "mux_multi_decode")
+
+
+def paged_decode(out, q, k_pool, v_pool, block_tables, context_lens, max_context_len, scale,
+                 layer: int = 0, partition_size: int = 0, workspace=None, stream=None) -> None:
+    multi_decode([DecodeCall(out, q, block_tables, context_lens, max_context_len, scale, layer)],
+                 k_pool, v_pool, partition_size, workspace, stream)
+
+
+def prefill_causal(out, q, k, v, cu_seqlens: torch.Tensor, max_prompt_len: int, scale: float,
+                   num_kv_heads: int, stream=None) -> None:
+    """Causal attention over packed prompts; cu_seqlens int32 [P+1] on the device."""
+    _need_cuda(out, q, k, v, cu_seqlens)
+    if cu_seqlens.dtype != torch.int32 or cu_seqlens.dim() != 1 or not cu_seqlens.is_contiguous():
+        raise ValueError("cu_seqlens: expected contiguous int32 [P+1]")
+    if q.shape[1] % HEAD_SIZE or k.shape[1] != num_kv_heads * HEAD_SIZE or k.shape != v.shape:
+        raise ValueError("q [T, Hq*128], k/v [T, Hkv*128] expected")
+    if not (q.dtype == k.dtype == v.dtype == out.dtype):
+        raise TypeError("q, k, v, out dtypes differ")
+    kv_stride = _rows(k, "k")
+    if _rows(v, "v") != kv_stride:
+        raise ValueError("k and v row strides differ")
+    rc = _lib.attn().mux_prefill_causal(
+        out.data_ptr(), _rows(out, "out"), q.data_ptr(), _rows(q, "q"), k.data_ptr(), v.data_ptr(), kv_stride,
+        cu_seqlens.data_ptr(), cu_seqlens.shape[0] - 1, int(max_prompt_len), q.shape[1] // HEAD_SIZE,
+        int(num_kv_heads), HEAD_SIZE, float(scale), _dtype_code(q), _stream_ptr(stream))
+    _lib.check_attn(rc, "mux_prefill_causal")

@@ -1,0 +1,290 @@
+"""GPU parity: KV-cache write (bit-exact) and paged decode attention (<= 2e-3
+max-abs, fp16/bf16 storage with fp32 accumulation) against the CPU oracle, all
+through the C ABI of libmuxattn.so.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import attn_oracle as orc
+from muxserve_amd import ops, workloads
+from muxserve_amd.pool import HEAD_SIZE, allocate_gpu_cache, num_gpu_blocks
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 2e-3   # max-abs bar of the decode path
+
+
+def _announce(msg):
+    print(f"[case] {msg}", flush=True)
+
+
+def _nan_pool(n, bs, dtype):
+    k, v = orc.allocate_pool(n, bs, dtype)
+    k.fill_(float("nan"))
+    v.fill_(float("nan"))
+    return k, v
+
+
+def _decode_case(seed, ctx_lens, Hq, Hkv, bs, dtype=torch.float16, partition=0, num_layers=1, layer=0,
+                 q_in_qkv=False, extra_blocks=7):
+    """Builds pool + tables on the host with the oracle's cache write, runs the
+    GPU decode, returns (gpu_out fp32, oracle_out fp32)."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    g = torch.Generator().manual_seed(seed)
+    B = len(ctx_lens)
+    ctx = np.asarray(ctx_lens, dtype=np.int32)
+    nblk = (ctx.astype(np.int64) + bs - 1) // bs
+    need = int(nblk.sum()) * Hkv
+    N = need + extra_blocks
+    ids = rng.permutation(N)[:need]
+    bt1, _ = workloads.build_tables(ctx, Hkv, bs, ids)
+    max_blocks = bt1.shape[-1]
+    bt = np.full((num_layers, B, Hkv, max_blocks), workloads.POISON_BLOCK, dtype=np.int32)
+    bt[layer] = bt1[0]
+    k_pool, v_pool = _nan_pool(N, bs, dtype)
+    # dense K/V per sequence -> written through the oracle's cache write
+    for s in range(B):
+        n = int(ctx[s])
+        kd = torch.randn((n, Hkv * HEAD_SIZE), generator=g).to(dtype)
+        vd = torch.randn((n, Hkv * HEAD_SIZE), generator=g).to(dtype)
+        i = np.arange(n)
+        slots = bt1[0, s][:, i // bs].astype(np.int64).T * bs + (i % bs)[:, None]     # [n, Hkv]
+        orc.reshape_and_cache(kd, vd, k_pool, v_pool, torch.from_numpy(slots[:, None, :]))
+    pad = (B + 7) // 8 * 8
+    if q_in_qkv:
+        qkv = torch.randn((pad, (Hq + 2 * Hkv) * HEAD_SIZE), generator=g).to(dtype)
+        q = qkv[:, :Hq * HEAD_SIZE]
+    else:
+        q = torch.randn((pad, Hq * HEAD_SIZE), generator=g).to(dtype)
+    scale = HEAD_SIZE ** -0.5
+    want = orc.paged_decode(q, k_pool, v_pool, torch.from_numpy(bt), ctx, scale, layer=layer)
+
+    dq = (qkv.to(DEV)[:, :Hq * HEAD_SIZE]) if q_in_qkv else q.to(DEV)
+    out = torch.full((pad, Hq * HEAD_SIZE), 7.0, dtype=dtype, device=DEV)
+    ops.paged_decode(out, dq, k_pool.to(DEV), v_pool.to(DEV), torch.from_numpy(bt).to(DEV),
+                     torch.from_numpy(ctx).to(DEV), int(ctx.max()), scale, layer=layer,
+                     partition_size=partition)
+    torch.cuda.synchronize()
+    got = out.float().cpu()
+    assert (got[B:] == 7.0).all(), "padding rows of out must not be written"
+    return got[:B], want
+
+
+def _check(got, want, tol=TOL, out_dtype=torch.float16):
+    """|got - want| <= 2e-3, plus, for bf16 outputs only, the rounding of the
+    result to its 8-bit mantissa (half an ulp = 2^-9 relative, taken as 2^-8
+    to cover values just below a power of two)."""
+    assert torch.isfinite(got).all()
+    bound = torch.full_like(want, tol)
+    if out_dtype == torch.bfloat16:
+        bound = bound + want.abs() * 2.0 ** -8
+    excess = ((got - want).abs() - bound).max().item()
+    err = (got - want).abs().max().item()
+    assert excess <= 0, f"max-abs error {err:.3e} exceeds {tol} (+ output rounding) by {excess:.3e}"
+    return err
+
+
+# ---- KV-cache write: bit-exact ---------------------------------------------------
+
+@pytest.mark.parametrize("bs", [16, 8, 32])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_reshape_and_cache_bit_exact_random_slots(bs, dtype):
+    _announce(f"reshape_and_cache random slots bs={bs} {dtype}")
+    rng = np.random.Generator(np.random.PCG64(bs))
+    g = torch.Generator().manual_seed(bs)
+    T, L, H, layer, N = 37, 3, 5, 1, 300
+    slots = rng.permutation(N * bs)[:T * L * H].reshape(T, L, H).astype(np.int64)
+    slots[3, layer, 2] = -1                      # skipped slot
+    pad = 40
+    qkv = torch.randn((pad, (H + 2 * H) * HEAD_SIZE), generator=g).to(dtype)
+    k = qkv[:, H * HEAD_SIZE:2 * H * HEAD_SIZE]
+    v = qkv[:, 2 * H * HEAD_SIZE:]
+    k_pool, v_pool = orc.allocate_pool(N, bs, dtype)
+    k_pool.copy_(torch.randn(k_pool.shape, generator=g).to(dtype))
+    v_pool.copy_(torch.randn(v_pool.shape, generator=g).to(dtype))
+    dk, dv = k_pool.to(DEV), v_pool.to(DEV)
+    dqkv = qkv.to(DEV)
+    ops.reshape_and_cache(dqkv[:, H * HEAD_SIZE:2 * H * HEAD_SIZE], dqkv[:, 2 * H * HEAD_SIZE:], dk, dv,
+                          torch.from_numpy(slots).to(DEV), layer=layer)
+    torch.cuda.synchronize()
+    orc.reshape_and_cache(k, v, k_pool, v_pool, torch.from_numpy(slots), layer=layer)
+    assert torch.equal(dk.cpu().view(torch.int16), k_pool.view(torch.int16))
+    assert torch.equal(dv.cpu().view(torch.int16), v_pool.view(torch.int16))
+
+
+def test_reshape_and_cache_prefill_pattern_roundtrip():
+    """Prompt-shaped slots (token i -> block i//bs, offset i%bs per head), then
+    gather back through the tables: gather(scatter(x)) == x bitwise."""
+    _announce("reshape_and_cache prefill roundtrip")
+    bs, H = 16, 4
+    rng = np.random.Generator(np.random.PCG64(5))
+    g = torch.Generator().manual_seed(5)
+    lens = np.array([1, 16, 17, 100, 31], dtype=np.int32)
+    N = 400
+    ids = rng.permutation(N)
+    slots, used = workloads.prefill_slot_mapping(lens, H, bs, ids)
+    T = int(lens.sum())
+    k = torch.randn((T, H * HEAD_SIZE), generator=g).half()
+    v = torch.randn((T, H * HEAD_SIZE), generator=g).half()
+    dk, dv = allocate_gpu_cache(N, bs, DEV)
+    dk.zero_()
+    dv.zero_()
+    ops.reshape_and_cache(k.to(DEV), v.to(DEV), dk, dv, torch.from_numpy(slots).to(DEV))
+    torch.cuda.synchronize()
+    hk, hv = dk.cpu(), dv.cpu()
+    start, cur = 0, 0
+    for n in lens:
+        n = int(n)
+        nblk = (n + bs - 1) // bs
+        blk = ids[cur:cur + nblk * H].reshape(nblk, H)
+        cur += nblk * H
+        for h in range(H):
+            K, V = orc.gather_kv(hk, hv, torch.from_numpy(blk[:, h].astype(np.int32)), n)
+            assert torch.equal(K, k[start:start + n, h * HEAD_SIZE:(h + 1) * HEAD_SIZE])
+            assert torch.equal(V, v[start:start + n, h * HEAD_SIZE:(h + 1) * HEAD_SIZE])
+        start += n
+
+
+# ---- paged decode ------------------------------------------------------------------
+
+def test_decode_config1_shape():
+    """7B layer, 32 heads, batch 8, ctx ~ U{64..512}, block size 16."""
+    _announce("decode config 1")
+    models, N = workloads.config1(seed=0)
+    m = models[0]
+    got, want = _decode_case(1, m.context_lens, 32, 32, 16)
+    _check(got, want)
+
+
+@pytest.mark.parametrize("ctx", [[1], [2, 15, 16, 17], [63, 64, 65, 127, 128, 129], [255, 256, 257, 300]])
+def test_decode_boundaries(ctx):
+    _announce(f"decode boundaries ctx={ctx}")
+    got, want = _decode_case(2, ctx, 4, 4, 16)
+    _check(got, want)
+
+
+@pytest.mark.parametrize("partition", [64, 128, 256, 512])
+def test_decode_split_context_equals_single_pass(partition):
+    _announce(f"decode split partition={partition}")
+    ctx = [1, 64, 65, 200, 513, 777, 1024, 1500]
+    got, want = _decode_case(3, ctx, 3, 3, 16, partition=partition)
+    _check(got, want)
+
+
+@pytest.mark.parametrize("bs", [8, 32])
+def test_decode_other_block_sizes(bs):
+    _announce(f"decode bs={bs}")
+    got, want = _decode_case(4, [1, 7, 8, 9, 31, 32, 33, 100, 400], 3, 3, bs, partition=128)
+    _check(got, want)
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(8, 4), (8, 2), (16, 2), (6, 2), (64, 8)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_decode_gqa(Hq, Hkv, dtype):
+    _announce(f"decode gqa Hq={Hq} Hkv={Hkv} {dtype}")
+    got, want = _decode_case(5, [5, 64, 130, 700], Hq, Hkv, 16, dtype=dtype, partition=256)
+    _check(got, want, out_dtype=dtype)
+
+
+def test_decode_layer_slice_and_strided_q():
+    """layer_idx selects block_tables[l]; q is a column slice of a qkv row."""
+    _announce("decode layer slice + strided q")
+    got, want = _decode_case(6, [40, 300, 17], 5, 5, 16, num_layers=3, layer=2, q_in_qkv=True)
+    _check(got, want)
+
+
+def test_decode_identical_keys_gives_mean_of_values():
+    _announce("decode identical keys")
+    bs, H, ctx = 16, 2, 150
+    N = 64
+    k_pool, v_pool = _nan_pool(N, bs, torch.float16)
+    g = torch.Generator().manual_seed(9)
+    key = torch.randn(H * HEAD_SIZE, generator=g).half()
+    vals = torch.randn((ctx, H * HEAD_SIZE), generator=g).half()
+    ids = np.arange(N)[::-1].copy()
+    bt, _ = workloads.build_tables([ctx], H, bs, ids)
+    i = np.arange(ctx)
+    slots = bt[0, 0][:, i // bs].astype(np.int64).T * bs + (i % bs)[:, None]
+    orc.reshape_and_cache(key.expand(ctx, -1).contiguous(), vals, k_pool, v_pool,
+                          torch.from_numpy(slots[:, None, :]))
+    q = torch.randn((8, H * HEAD_SIZE), generator=g).half()
+    out = torch.zeros((8, H * HEAD_SIZE), dtype=torch.float16, device=DEV)
+    ops.paged_decode(out, q.to(DEV), k_pool.to(DEV), v_pool.to(DEV), torch.from_numpy(bt).to(DEV),
+                     torch.tensor([ctx], dtype=torch.int32, device=DEV), ctx, HEAD_SIZE ** -0.5,
+                     partition_size=64)
+    torch.cuda.synchronize()
+    _check(out[:1].float().cpu(), vals.float().mean(dim=0, keepdim=True))
+
+
+def test_multi_decode_three_models_one_launch_matches_separate_launches():
+    _announce("multi decode 3 models")
+    bs = 16
+    models, need = workloads.config2(seed=3, num_pool_blocks=20000, batches=(6, 4, 3))
+    N = 20000
+    dk, dv = allocate_gpu_cache(N, bs, DEV)
+    dk.fill_(float("nan"))
+    dv.fill_(float("nan"))
+    used = np.concatenate([m.used_blocks(bs) for m in models])
+    assert len(np.unique(used)) == len(used) == need
+    workloads.fill_blocks(dk, dv, used, seed=3)
+    for i, m in enumerate(models):
+        m.to_device(DEV, torch.float16, seed=10 + i)
+    calls = [ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale)
+             for m in models]
+    ops.multi_decode(calls, dk, dv, partition_size=256)
+    torch.cuda.synchronize()
+    fused = [m.out.clone() for m in models]
+    for m in models:
+        m.out.zero_()
+        ops.paged_decode(m.out, m.q, dk, dv, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                         partition_size=256)
+    torch.cuda.synchronize()
+    ks, vs, tables = workloads.compact_to_host(dk, dv, models, bs)
+    for m, f, t in zip(models, fused, tables):
+        assert torch.equal(f, m.out), "fused and separate launches must agree bitwise"
+        want = orc.paged_decode(m.q.cpu(), ks, vs, t, m.context_lens, m.scale)
+        _check(f[:m.batch].float().cpu(), want)
+
+
+def test_decode_rejects_bad_arguments():
+    _announce("decode argument validation")
+    dk, dv = allocate_gpu_cache(8, 16, DEV)
+    q = torch.zeros((8, 256), dtype=torch.float16, device=DEV)
+    out = torch.zeros_like(q)
+    bt = torch.zeros((1, 2, 2, 4), dtype=torch.int32, device=DEV)
+    cl = torch.ones(2, dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError):   # max_context_len exceeds what a table row can hold
+        ops.paged_decode(out, q, dk, dv, bt, cl, 4 * 16 + 1, 1.0)
+    with pytest.raises(RuntimeError):   # partition must be a multiple of 64
+        ops.paged_decode(out, q, dk, dv, bt, cl, 16, 1.0, partition_size=100)
+    with pytest.raises(RuntimeError):   # CPU tensors: there is no CPU path
+        ops.paged_decode(out.cpu(), q.cpu(), dk, dv, bt, cl, 16, 1.0)
+    torch.cuda.synchronize()
+
+
+def test_decode_config2_full_size_pool():
+    """Headline workload at its real size: pool = 60% of HBM, three models,
+    ids scattered over the whole pool.  Checked against the oracle on a compact
+    host copy of the referenced blocks (attention is invariant under relabelling
+    physical blocks)."""
+    _announce("decode config 2 full size")
+    bs = 16
+    total = torch.cuda.get_device_properties(0).total_memory
+    N = num_gpu_blocks(0.6, total, bs)
+    dk, dv = allocate_gpu_cache(N, bs, DEV)
+    models, need = workloads.config2(seed=0, num_pool_blocks=N)
+    used = np.concatenate([m.used_blocks(bs) for m in models])
+    assert used.max() > N // 2, "ids must span the pool"
+    workloads.fill_blocks(dk, dv, used, seed=0)
+    for i, m in enumerate(models):
+        m.to_device(DEV, torch.float16, seed=20 + i)
+    calls = [ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale)
+             for m in models]
+    ops.multi_decode(calls, dk, dv)
+    torch.cuda.synchronize()
+    ks, vs, tables = workloads.compact_to_host(dk, dv, models, bs)
+    del dk, dv
+    for m, t in zip(models, tables):
+        want = orc.paged_decode(m.q.cpu(), ks, vs, t, m.context_lens, m.scale)
+        _check(m.out[:m.batch].float().cpu(), want)
