@@ -49,6 +49,9 @@ extern "C" {
 #define MUXA_DTYPE_BF16 1
 
 #define MUXA_MAX_DECODE_ITEMS 8
+/* Leading region of a decode workspace: int32 arrival counters, one per
+ * (sequence, group of query heads sharing a wave) over all items of a call. */
+#define MUXA_DECODE_COUNTER_BYTES (1u << 20)
 
 /* Library version (major*10000 + minor*100 + patch). */
 int32_t mux_attn_version(void);
@@ -85,9 +88,17 @@ int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t kv_row_strid
  * context_lens: int32 [num_seqs].  max_context_len: host-side upper bound on
  * context_lens (InputMetadata.max_context_len, pipeworker.py:81-90); it sizes
  * the grid, device values above it are clamped.
+ * total_context_len: optional host-side upper bound on the sum of
+ * context_lens (the serving loop has them on the host before the copy,
+ * llm_runtime.py:311-326); it only tightens the grid, 0 = unknown.
  * partition_size: tokens per split of a context (multiple of 64), 0 = choose.
  * workspace: scratch for split partials, at least
- * mux_paged_decode_workspace_bytes(...) bytes; may be NULL when that is 0. */
+ * mux_paged_decode_workspace_bytes(...) bytes, 16-byte aligned; may be NULL
+ * when that is 0.  Its first MUXA_DECODE_COUNTER_BYTES bytes are arrival
+ * counters that must be ZERO when a launch begins: zero them once with
+ * mux_paged_decode_workspace_init (or any fill) before first use; every
+ * completed launch leaves them zero again.  Launches that share a workspace
+ * must not overlap. */
 typedef struct MuxDecodeItem {
   void *out;
   const void *q;
@@ -95,6 +106,7 @@ typedef struct MuxDecodeItem {
   int64_t q_row_stride;
   const int32_t *block_tables;   /* base of the [L, B, Hkv, max_blocks] tensor */
   const int32_t *context_lens;
+  int64_t total_context_len;     /* host-side upper bound on sum(context_lens); 0 = unknown */
   int32_t layer;
   int32_t num_layers;
   int32_t num_seqs;
@@ -107,6 +119,10 @@ typedef struct MuxDecodeItem {
 
 size_t mux_paged_decode_workspace_bytes(const MuxDecodeItem *items, int32_t n_items,
                                         int32_t partition_size);
+
+/* Zero-fills the counter region of a decode workspace (a fill kernel on
+ * `stream`, safe to capture). */
+int32_t mux_paged_decode_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
 
 /* Fused launch over up to MUXA_MAX_DECODE_ITEMS models that share the pool,
  * head size, block size and dtype ("mixed multi-LLM decode": one grid covers

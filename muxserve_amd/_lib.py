@@ -7,8 +7,10 @@ import ctypes
 import os
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-HOST_LIB_PATH = os.path.join(_PKG, "libmuxhost.so")
-ATTN_LIB_PATH = os.path.join(_PKG, "libmuxattn.so")
+# The in-tree builds; the environment variables let a developer point at an
+# alternative build of the same ABI (e.g. one compiled with other flags).
+HOST_LIB_PATH = os.environ.get("MUXSERVE_HOST_LIB", os.path.join(_PKG, "libmuxhost.so"))
+ATTN_LIB_PATH = os.environ.get("MUXSERVE_ATTN_LIB", os.path.join(_PKG, "libmuxattn.so"))
 
 _host = None
 _attn = None
@@ -101,6 +103,7 @@ class MuxDecodeItem(ctypes.Structure):
         ("out", c_vp), ("q", c_vp),
         ("out_row_stride", c_i64), ("q_row_stride", c_i64),
         ("block_tables", c_vp), ("context_lens", c_vp),
+        ("total_context_len", c_i64),
         ("layer", c_i32), ("num_layers", c_i32), ("num_seqs", c_i32),
         ("num_q_heads", c_i32), ("num_kv_heads", c_i32),
         ("max_blocks", c_i32), ("max_context_len", c_i32),
@@ -114,6 +117,7 @@ ATTN_SIGNATURES = {
     "mux_reshape_and_cache": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i32, c_i32,
                                       c_i32, c_i32, c_i32, c_i32, c_i32, c_vp]),
     "mux_paged_decode_workspace_bytes": (c_sz, [c_vp, c_i32, c_i32]),
+    "mux_paged_decode_workspace_init": (c_i32, [c_vp, c_sz, c_vp]),
     "mux_multi_decode": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_i32,
                                  c_vp, c_sz, c_vp]),
     "mux_paged_decode": (c_i32, [c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_vp,

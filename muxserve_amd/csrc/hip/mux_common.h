@@ -121,4 +121,21 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Inclusive prefix sum over the 64 lanes of a wave (row shifts, then the two
+// cross-row broadcasts of the GCN/CDNA DPP unit).  Lanes whose DPP source is
+// outside the row or masked off receive 0.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ int dpp_or_zero(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, kCtrl, kRowMask, 0xf, false);
+}
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+  v += dpp_or_zero<0x111, 0xf>(v);   // row_shr:1
+  v += dpp_or_zero<0x112, 0xf>(v);   // row_shr:2
+  v += dpp_or_zero<0x114, 0xf>(v);   // row_shr:4
+  v += dpp_or_zero<0x118, 0xf>(v);   // row_shr:8
+  v += dpp_or_zero<0x142, 0xa>(v);   // row_bcast:15 -> rows 1 and 3
+  v += dpp_or_zero<0x143, 0xc>(v);   // row_bcast:31 -> rows 2 and 3
+  return v;
+}
+
 }  // namespace mux

@@ -1,8 +1,8 @@
 // Paged decode attention over the head-granular KV pool, gfx950.
 //
-// Work unit = one wave64 = (model, sequence, group of G query heads that share
-// a kv head, partition of the context).  A wave walks its partition in tiles
-// of 64 tokens:
+// Work unit = (model, sequence, group of G query heads that share a kv head,
+// partition of the context).  A workgroup of NW waves handles one unit at a
+// time; wave w takes tiles w, w+NW, ... of 64 tokens:
 //   * K: lane t owns token t of the tile.  Pool layout [D/8][BS][8] makes the
 //     8 dims of one token a 16-byte chunk; 16 loads (one per d/8) bring the
 //     token's whole key into 64 VGPRs, each load instruction reading whole
@@ -16,15 +16,22 @@
 //     each lane accumulates BS/4 output dims, partial over its 8 tokens; the
 //     BS/8 partials per dim are summed once at the end with DPP.
 // All 32 loads of a tile (16 KiB K + 16 KiB V per wave) are issued before the
-// first use, which is what keeps HBM busy; arithmetic is <15% of VALU time.
+// first use; the waves' partial results meet in LDS and wave 0 merges them.
 //
-// Contexts longer than `partition` tokens are split; partials (max, sum,
-// unnormalised acc) go to the workspace and a second small kernel combines
-// them.  Sequences that fit one partition write their output directly.
+// Contexts longer than `partition` tokens are split; each partition's partial
+// (max, sum, unnormalised acc) goes to the workspace and the workgroup that
+// arrives LAST for a (sequence, head group) - found with one atomic counter per
+// group - combines them and writes the output, so a step is a single kernel.
+// Sequences that fit one partition write their output directly.
+//
+// Units are enumerated compactly from the device-side context lengths (a
+// wave-wide prefix sum), so the grid holds (almost) no empty workgroups; per
+// model the split sequences come first and the sequences that need no combine
+// last, which keeps the kernel's tail short.
 //
 // Several models (different head counts, tables, q/out tensors) are covered by
 // one grid: the kernel argument carries up to MUXA_MAX_DECODE_ITEMS item
-// descriptors and each wave finds its item from its block index.
+// descriptors.
 #include "mux_common.h"
 
 #include <algorithm>
@@ -32,6 +39,8 @@
 namespace mux {
 
 thread_local int32_t g_last_hip_error = 0;
+
+constexpr int kWavesPerGroup = 4;         // waves cooperating on one unit
 
 struct DecodeItemDev {
   void *out;
@@ -41,10 +50,10 @@ struct DecodeItemDev {
   const int32_t *ctx;             // [B]
   float *ws_acc;                  // [B, Hq, max_splits, 128]
   float *ws_ml;                   // [B, Hq, max_splits, 2]  (running max in log2 units, sum)
+  int32_t *counters;              // [B, Hq/G] arrivals per (sequence, head group); zero between launches
   int32_t B, Hq, Hkv, ratio;      // ratio = Hq / Hkv
   int32_t max_blocks, max_splits, max_ctx;
-  int32_t work_begin;             // first block of this item in the main grid
-  int32_t row_begin;              // first (seq, hq) row of this item in the reduce grid
+  int32_t work_begin;             // first block of this item in the grid
   float scale_log2;               // scale * log2(e)
 };
 
@@ -57,19 +66,359 @@ struct DecodeParams {
   int32_t last_block;             // num_pool_blocks - 1: table entries are clamped to it
 };
 
-template <typename T, int BS, int G>
-__global__ __launch_bounds__(64) void paged_decode_kernel(const DecodeParams P) {
-  constexpr int D = kHeadSize;
-  constexpr int BPT = 64 / BS;               // blocks per tile
-  constexpr int PARTS = BS / 8;              // 16-byte chunks per V row of a block
-  constexpr int VI = D * PARTS / 64;         // V load instructions per block
-  constexpr int BLOCK_CHUNKS = D * BS / 8;   // 16-byte chunks per K block (same for V)
+// One unit of work, uniform across the workgroup.
+struct Unit {
+  int item, seq, split, ctx, wh, t0, t1;
+};
+
+// Device-coherent accesses for data handed between workgroups of one kernel
+// that may run on different XCDs (each XCD has its own L2).
+__device__ __forceinline__ void coherent_store(float *p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float coherent_load(const float *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Orders a wave's own LDS writes before its following LDS reads of data other
+// lanes wrote.  One wave's LDS instructions execute in order, so this only has
+// to stop the compiler from moving them.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int BS>
+struct Geometry {
   static_assert(BS == 8 || BS == 16 || BS == 32, "block size");
+  static constexpr int D = kHeadSize;
+  static constexpr int BPT = 64 / BS;               // blocks per 64-token tile
+  static constexpr int PARTS = BS / 8;              // 16-byte chunks per V row of a block
+  static constexpr int VI = D * PARTS / 64;         // V load instructions per block
+  static constexpr int BLOCK_CHUNKS = D * BS / 8;   // 16-byte chunks per K block (same for V)
+};
 
-  __shared__ __attribute__((aligned(16))) float p_lds[G][64];
-  __shared__ __attribute__((aligned(16))) uint32_t q_lds[G][64];
+// This lane's block id for token tb+lane of a sequence's table row (0 for
+// tokens at or past t1).  Clamped so that a corrupt table entry reads the
+// wrong block instead of faulting the GPU.
+template <int BS>
+__device__ __forceinline__ int load_block_id(const int32_t *trow, int tb, int t1, int lane, int last_block) {
+  const int tok = tb + lane;
+  int id = 0;
+  if (tok < t1) id = min(max(trow[tok / BS], 0), last_block);
+  return id;
+}
 
-  const int lane = threadIdx.x;
+// Issues every load of a tile: 16 K chunks for this lane's token, BPT*VI V chunks.
+template <int BS>
+__device__ __forceinline__ void issue_tile_loads(uint4 (&kreg)[16], uint4 (&vreg)[Geometry<BS>::BPT][Geometry<BS>::VI],
+                                                 const uint4 *kpool, const uint4 *vpool, int id, int tb, int t1,
+                                                 int lane) {
+  using Geo = Geometry<BS>;
+  const int tok = tb + lane;
+  const int part = lane % Geo::PARTS;
+  if (tok < t1) {
+    const uint4 *kp = kpool + static_cast<int64_t>(id) * Geo::BLOCK_CHUNKS + (tok % BS);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) kreg[j] = kp[j * BS];
+  } else {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) kreg[j] = make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int b = 0; b < Geo::BPT; ++b) {
+    const int idb = __builtin_amdgcn_readlane(id, b * BS);   // the block's id, uniform
+    const uint4 *vp = vpool + static_cast<int64_t>(idb) * Geo::BLOCK_CHUNKS + lane;
+    const bool chunk_ok = tb + b * BS + part * 8 < t1;
+#pragma unroll
+    for (int j = 0; j < Geo::VI; ++j) {
+      if (chunk_ok) vreg[b][j] = vp[j * 64];
+      else vreg[b][j] = make_uint4(0, 0, 0, 0);
+    }
+  }
+}
+
+// Scores, online softmax and P.V for one loaded tile.
+template <typename T, int BS, int G>
+__device__ __forceinline__ void consume_tile(uint4 (&kreg)[16], uint4 (&vreg)[Geometry<BS>::BPT][Geometry<BS>::VI],
+                                             const uint32_t (&q_s)[64], const uint32_t (*q_w)[64],
+                                             float (*p_w)[64], float (&m)[G], float (&l)[G],
+                                             float (&acc)[G][Geometry<BS>::VI], float scale_log2, int tb, int t1,
+                                             int lane) {
+  using Geo = Geometry<BS>;
+  const int part = lane % Geo::PARTS;
+  const bool valid = tb + lane < t1;
+  // Tail tile: zero V elements of tokens >= t1 (their probability is 0 but
+  // the slots were never written and may hold NaN/Inf bit patterns).
+  if (tb + 64 > t1) {
+#pragma unroll
+    for (int b = 0; b < Geo::BPT; ++b) {
+      const int n_ok = t1 - (tb + b * BS + part * 8);   // valid tokens in this lane's chunk
+#pragma unroll
+      for (int j = 0; j < Geo::VI; ++j) {
+        uint32_t *wv = reinterpret_cast<uint32_t *>(&vreg[b][j]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (2 * e >= n_ok) wv[e] = 0u;
+          else if (2 * e + 1 >= n_ok) wv[e] &= 0x0000ffffu;
+        }
+      }
+    }
+  }
+
+  float s[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      uint4 qq;
+      if constexpr (G == 1) qq = make_uint4(q_s[4 * j], q_s[4 * j + 1], q_s[4 * j + 2], q_s[4 * j + 3]);
+      else qq = reinterpret_cast<const uint4 *>(q_w[g])[j];
+      a0 = dot2<T>(kreg[j].x, qq.x, a0);
+      a1 = dot2<T>(kreg[j].y, qq.y, a1);
+      a0 = dot2<T>(kreg[j].z, qq.z, a0);
+      a1 = dot2<T>(kreg[j].w, qq.w, a1);
+    }
+    s[g] = valid ? (a0 + a1) * scale_log2 : -INFINITY;
+  }
+
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const float m_new = fmaxf(m[g], wave_max(s[g]));
+    const float alpha = fast_exp2(m[g] - m_new);
+    const float p = fast_exp2(s[g] - m_new);
+    l[g] = l[g] * alpha + p;
+#pragma unroll
+    for (int j = 0; j < Geo::VI; ++j) acc[g][j] *= alpha;
+    m[g] = m_new;
+    p_w[g][lane] = p;
+  }
+  wave_lds_sync();
+
+#pragma unroll
+  for (int b = 0; b < Geo::BPT; ++b) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const float4 pa = *reinterpret_cast<const float4 *>(&p_w[g][b * BS + part * 8]);
+      const float4 pb = *reinterpret_cast<const float4 *>(&p_w[g][b * BS + part * 8 + 4]);
+#pragma unroll
+      for (int j = 0; j < Geo::VI; ++j) {
+        float a = acc[g][j];
+        a = fma2<T>(vreg[b][j].x, pa.x, pa.y, a);
+        a = fma2<T>(vreg[b][j].y, pa.z, pa.w, a);
+        a = fma2<T>(vreg[b][j].z, pb.x, pb.y, a);
+        a = fma2<T>(vreg[b][j].w, pb.z, pb.w, a);
+        acc[g][j] = a;
+      }
+    }
+  }
+  wave_lds_sync();
+}
+
+// This wave's partial (a wave without tiles contributes max=-inf, sum=0) to LDS.
+template <int BS, int G>
+__device__ __forceinline__ void stash_wave_partial(float (&m)[G], float (&l)[G], float (&acc)[G][Geometry<BS>::VI],
+                                                   float (*xa)[kHeadSize], float (*xm)[2], int lane) {
+  using Geo = Geometry<BS>;
+  const int part = lane % Geo::PARTS;
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const float L = wave_sum(l[g]);
+#pragma unroll
+    for (int j = 0; j < Geo::VI; ++j) {
+      float a = acc[g][j];
+      if constexpr (Geo::PARTS >= 2) a += dpp_mov<0xB1>(a);
+      if constexpr (Geo::PARTS >= 4) a += dpp_mov<0x4E>(a);
+      const int d = j * (64 / Geo::PARTS) + lane / Geo::PARTS;
+      if (part == 0) xa[g][d] = a;
+    }
+    if (lane == 0) {
+      xm[g][0] = m[g];
+      xm[g][1] = L;
+    }
+  }
+}
+
+// Wave 0: merge the workgroup's NW partials (lane owns dims lane and lane+64),
+// then either write the output (context fits one partition) or publish the
+// partition's partial and, if this was the last partition to arrive, combine
+// them all.
+template <typename T, int G, int NW>
+__device__ __forceinline__ void merge_and_write(const DecodeItemDev &I, const Unit &u, int partition,
+                                                const float (*xa)[G][kHeadSize], const float (*xm)[G][2],
+                                                int lane) {
+  constexpr int D = kHeadSize;
+  const bool single = u.ctx <= partition;
+  const int hq0 = u.wh * G;
+#pragma unroll 1
+  for (int g = 0; g < G; ++g) {
+    float M = xm[0][g][0];
+#pragma unroll
+    for (int k = 1; k < NW; ++k) M = fmaxf(M, xm[k][g][0]);
+    float L = 0.f, a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int k = 0; k < NW; ++k) {
+      const float wgt = fast_exp2(xm[k][g][0] - M);
+      L += xm[k][g][1] * wgt;
+      a0 += xa[k][g][lane] * wgt;
+      a1 += xa[k][g][64 + lane] * wgt;
+    }
+    const int hq = hq0 + g;
+    if (single) {
+      uint16_t *o = static_cast<uint16_t *>(I.out) + static_cast<int64_t>(u.seq) * I.out_stride + hq * D;
+      o[lane] = to_storage<T>(a0 / L);
+      o[64 + lane] = to_storage<T>(a1 / L);
+    } else {
+      const int64_t prow = (static_cast<int64_t>(u.seq) * I.Hq + hq) * I.max_splits + u.split;
+      coherent_store(&I.ws_acc[prow * D + lane], a0);
+      coherent_store(&I.ws_acc[prow * D + 64 + lane], a1);
+      if (lane == 0) {
+        coherent_store(&I.ws_ml[prow * 2], M);
+        coherent_store(&I.ws_ml[prow * 2 + 1], L);
+      }
+    }
+  }
+  if (single) return;
+
+  // Partials are written and read with device-coherent accesses (they bypass
+  // the per-XCD L2), so ordering them against the arrival counter needs only
+  // "my stores have completed" / "my loads issue after the atomic returned" -
+  // a workgroup-scope fence, i.e. a wait, not an L2 write-back/invalidate.
+  const int n_splits = (u.ctx + partition - 1) / partition;
+  int32_t *counter = I.counters + static_cast<int64_t>(u.seq) * (I.Hq / G) + u.wh;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  int arrived = 0;
+  if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  arrived = __builtin_amdgcn_readfirstlane(arrived);
+  if (arrived != n_splits - 1) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll 1
+  for (int g = 0; g < G; ++g) {
+    const int hq = hq0 + g;
+    const int64_t base = (static_cast<int64_t>(u.seq) * I.Hq + hq) * I.max_splits;
+    const float *ml = I.ws_ml + base * 2;
+    const float *pa = I.ws_acc + base * D;
+    float M = -INFINITY;
+    for (int i = 0; i < n_splits; ++i) M = fmaxf(M, coherent_load(&ml[i * 2]));
+    float Lsum = 0.f, a0 = 0.f, a1 = 0.f;
+    for (int i = 0; i < n_splits; ++i) {
+      const float wgt = fast_exp2(coherent_load(&ml[i * 2]) - M);
+      Lsum += coherent_load(&ml[i * 2 + 1]) * wgt;
+      a0 += coherent_load(&pa[i * D + lane]) * wgt;
+      a1 += coherent_load(&pa[i * D + 64 + lane]) * wgt;
+    }
+    uint16_t *o = static_cast<uint16_t *>(I.out) + static_cast<int64_t>(u.seq) * I.out_stride + hq * D;
+    o[lane] = to_storage<T>(a0 / Lsum);
+    o[64 + lane] = to_storage<T>(a1 / Lsum);
+  }
+  // Ready for the next launch.
+  if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---------------------------------------------------------------------------
+// Direct kernel: one workgroup per unit, unit found by scanning the context
+// lengths in global memory.
+// ---------------------------------------------------------------------------
+
+// Maps pair index e to (sequence, partition index).  Every lane returns the
+// same answer; false: e is past the last pair (grid padding).  Pairs are
+// numbered in three classes, chosen so that the kernel's last workgroups are
+// the ones that finish fastest:
+//   1. the remainder (ctx % partition tokens) of every sequence longer than one
+//      partition - dispatched first, so the partition that arrives last and
+//      combines a split sequence is normally a full one in mid-kernel;
+//   2. all full partitions of those sequences;
+//   3. sequences that fit one partition (ctx <= partition): no partials, no
+//      atomics, the output is written straight from the workgroup.
+__device__ __forceinline__ bool locate_pair_global(const int32_t *ctx_arr, int B, int max_ctx, int partition,
+                                                   int e, int lane, int &seq, int &split, int &ctx) {
+  int base = 0;
+  // class 1: remainders of split sequences
+  for (int c0 = 0; c0 < B; c0 += 64) {
+    const int s = c0 + lane;
+    const int c = s < B ? max(min(ctx_arr[s], max_ctx), 0) : 0;
+    const bool hit_class = c > partition && (c % partition) != 0;
+    const unsigned long long mask = __builtin_amdgcn_ballot_w64(hit_class);
+    const int cnt = __popcll(mask);
+    if (e < base + cnt) {
+      const int upto = __popcll(mask & (~0ull >> (63 - lane)));     // class members in lanes 0..lane
+      const unsigned long long hit = __builtin_amdgcn_ballot_w64(hit_class && upto == e - base + 1);
+      const int k = __ffsll(static_cast<long long>(hit)) - 1;
+      seq = c0 + k;
+      ctx = __builtin_amdgcn_readlane(c, k);
+      split = ctx / partition;
+      return true;
+    }
+    base += cnt;
+  }
+  // class 2: full partitions of split sequences
+  for (int c0 = 0; c0 < B; c0 += 64) {
+    const int s = c0 + lane;
+    const int c = s < B ? max(min(ctx_arr[s], max_ctx), 0) : 0;
+    const int full = c > partition ? c / partition : 0;
+    const int incl = wave_inclusive_scan(full);
+    const int total = __builtin_amdgcn_readlane(incl, 63);
+    if (e < base + total) {
+      const int k = __popcll(__builtin_amdgcn_ballot_w64(base + incl <= e));
+      seq = c0 + k;
+      split = e - base - __builtin_amdgcn_readlane(incl - full, k);
+      ctx = __builtin_amdgcn_readlane(c, k);
+      return true;
+    }
+    base += total;
+  }
+  // class 3: sequences that fit one partition
+  for (int c0 = 0; c0 < B; c0 += 64) {
+    const int s = c0 + lane;
+    const int c = s < B ? max(min(ctx_arr[s], max_ctx), 0) : 0;
+    const bool hit_class = c > 0 && c <= partition;
+    const unsigned long long mask = __builtin_amdgcn_ballot_w64(hit_class);
+    const int cnt = __popcll(mask);
+    if (e < base + cnt) {
+      const int upto = __popcll(mask & (~0ull >> (63 - lane)));
+      const unsigned long long hit = __builtin_amdgcn_ballot_w64(hit_class && upto == e - base + 1);
+      const int k = __ffsll(static_cast<long long>(hit)) - 1;
+      seq = c0 + k;
+      ctx = __builtin_amdgcn_readlane(c, k);
+      split = 0;
+      return true;
+    }
+    base += cnt;
+  }
+  return false;
+}
+
+// q of the unit's head group for the tile code.  G == 1: one coalesced 256-byte
+// load, then 64 readlanes make it uniform (SGPRs) so q.k needs no q registers
+// per lane.  G > 1: this wave's LDS copy.
+template <int G>
+__device__ __forceinline__ void fetch_q(const DecodeItemDev &I, int seq, int hq0, int lane, uint32_t (&q_s)[64],
+                                        uint32_t (*q_w)[64]) {
+  const uint32_t *qv = reinterpret_cast<const uint32_t *>(
+      static_cast<const uint16_t *>(I.q) + static_cast<int64_t>(seq) * I.q_stride + hq0 * kHeadSize);
+  if constexpr (G == 1) {
+    const uint32_t mine = qv[lane];
+#pragma unroll
+    for (int i = 0; i < 64; ++i) q_s[i] = __builtin_amdgcn_readlane(mine, i);
+  } else {
+#pragma unroll
+    for (int g = 0; g < G; ++g) q_w[g][lane] = qv[g * 64 + lane];
+    wave_lds_sync();
+  }
+}
+
+template <typename T, int BS, int G, int NW>
+__global__ __launch_bounds__(64 * NW) void paged_decode_kernel(const DecodeParams P) {
+  using Geo = Geometry<BS>;
+  __shared__ __attribute__((aligned(16))) float p_lds[NW][G][64];     // per-wave probabilities of a tile
+  __shared__ __attribute__((aligned(16))) uint32_t q_lds[NW][G][64];  // G > 1: per-wave copy of the group's q
+  __shared__ float x_acc[NW][G][kHeadSize];                           // per-wave partial outputs
+  __shared__ float x_ml[NW][G][2];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int w = blockIdx.x;
   int ii = 0;
 #pragma unroll
@@ -77,208 +426,53 @@ __global__ __launch_bounds__(64) void paged_decode_kernel(const DecodeParams P) 
     if (k < P.n_items && w >= P.it[k].work_begin) ii = k;
   const DecodeItemDev &I = P.it[ii];
 
-  const int WH = I.Hq / G;                   // work heads per sequence
+  const int WH = I.Hq / G;                   // head groups per sequence
   const int local = w - I.work_begin;
-  const int per_split = I.B * WH;
-  const int split = local / per_split;
-  const int r = local - split * per_split;
-  const int seq = r / WH;
-  const int wh = r - seq * WH;
-  const int hq0 = wh * G;
-  const int hk = hq0 / I.ratio;
-  const int ctx = min(I.ctx[seq], I.max_ctx);
+  const int e = local / WH;
+  Unit u;
+  u.item = ii;
+  u.wh = local - e * WH;
   const int partition = P.partition;
-  const int t0 = split * partition;
-  if (t0 >= ctx) return;
-  const int t1 = min(ctx, t0 + partition);
-  const bool single = ctx <= partition;
+  // Every wave of the workgroup derives the same unit (or all of them leave).
+  if (!locate_pair_global(I.ctx, I.B, I.max_ctx, partition, e, lane, u.seq, u.split, u.ctx)) return;
+  u.t0 = u.split * partition;
+  u.t1 = min(u.ctx, u.t0 + partition);
+  const int hq0 = u.wh * G;
+  const int hk = hq0 / I.ratio;
 
-  // ---- q: 128 dims = 64 packed pairs per head --------------------------------
-  const uint32_t *qrow = reinterpret_cast<const uint32_t *>(
-      static_cast<const uint16_t *>(I.q) + static_cast<int64_t>(seq) * I.q_stride + hq0 * D);
-  uint32_t q_s[64];   // G == 1: the head's q, uniform across lanes (lives in SGPRs)
-  if constexpr (G == 1) {
-    const uint32_t qv = qrow[lane];
-#pragma unroll
-    for (int i = 0; i < 64; ++i) q_s[i] = __builtin_amdgcn_readlane(qv, i);
-  } else {
-#pragma unroll
-    for (int g = 0; g < G; ++g) q_lds[g][lane] = qrow[g * 64 + lane];
-    __syncthreads();
-  }
+  uint32_t q_s[64];
+  fetch_q<G>(I, u.seq, hq0, lane, q_s, q_lds[wave]);
 
-  const int32_t *trow = I.tables + (static_cast<int64_t>(seq) * I.Hkv + hk) * I.max_blocks;
+  const int32_t *trow = I.tables + (static_cast<int64_t>(u.seq) * I.Hkv + hk) * I.max_blocks;
   const uint4 *kpool = static_cast<const uint4 *>(P.k_pool);
   const uint4 *vpool = static_cast<const uint4 *>(P.v_pool);
-  const float scale_log2 = I.scale_log2;
-  const int part = lane % PARTS;
 
-  float m[G], l[G], acc[G][VI];
+  float m[G], l[G], acc[G][Geo::VI];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     m[g] = -INFINITY;
     l[g] = 0.f;
 #pragma unroll
-    for (int j = 0; j < VI; ++j) acc[g][j] = 0.f;
+    for (int j = 0; j < Geo::VI; ++j) acc[g][j] = 0.f;
   }
-
-  for (int tb = t0; tb < t1; tb += 64) {
-    const int tok = tb + lane;
-    const bool valid = tok < t1;
-    int id = 0;
-    // Clamp so that a corrupt table entry reads the wrong block instead of
-    // faulting the GPU.
-    if (valid) id = min(max(trow[tok / BS], 0), P.last_block);
-
-    // ---- issue every load of the tile ---------------------------------------
+  for (int tb = u.t0 + wave * 64; tb < u.t1; tb += 64 * NW) {
+    const int id = load_block_id<BS>(trow, tb, u.t1, lane, P.last_block);
     uint4 kreg[16];
-    if (valid) {
-      const uint4 *kp = kpool + static_cast<int64_t>(id) * BLOCK_CHUNKS + (tok % BS);
-#pragma unroll
-      for (int j = 0; j < 16; ++j) kreg[j] = kp[j * BS];
-    } else {
-#pragma unroll
-      for (int j = 0; j < 16; ++j) kreg[j] = make_uint4(0, 0, 0, 0);
-    }
-    uint4 vreg[BPT][VI];
-#pragma unroll
-    for (int b = 0; b < BPT; ++b) {
-      const int idb = __builtin_amdgcn_readlane(id, b * BS);
-      const uint4 *vp = vpool + static_cast<int64_t>(idb) * BLOCK_CHUNKS + lane;
-      const bool chunk_ok = tb + b * BS + part * 8 < t1;
-#pragma unroll
-      for (int j = 0; j < VI; ++j) {
-        if (chunk_ok) vreg[b][j] = vp[j * 64];
-        else vreg[b][j] = make_uint4(0, 0, 0, 0);
-      }
-    }
-    // Tail tile: zero V elements of tokens >= t1 (their probability is 0 but
-    // the slots were never written and may hold NaN/Inf bit patterns).
-    if (tb + 64 > t1) {
-#pragma unroll
-      for (int b = 0; b < BPT; ++b) {
-        const int n_ok = t1 - (tb + b * BS + part * 8);   // valid tokens in this lane's chunk
-#pragma unroll
-        for (int j = 0; j < VI; ++j) {
-          uint32_t *wv = reinterpret_cast<uint32_t *>(&vreg[b][j]);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (2 * e >= n_ok) wv[e] = 0u;
-            else if (2 * e + 1 >= n_ok) wv[e] &= 0x0000ffffu;
-          }
-        }
-      }
-    }
-
-    // ---- scores ---------------------------------------------------------------
-    float s[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float a0 = 0.f, a1 = 0.f;
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        uint4 qq;
-        if constexpr (G == 1) qq = make_uint4(q_s[4 * j], q_s[4 * j + 1], q_s[4 * j + 2], q_s[4 * j + 3]);
-        else qq = reinterpret_cast<const uint4 *>(q_lds[g])[j];
-        a0 = dot2<T>(kreg[j].x, qq.x, a0);
-        a1 = dot2<T>(kreg[j].y, qq.y, a1);
-        a0 = dot2<T>(kreg[j].z, qq.z, a0);
-        a1 = dot2<T>(kreg[j].w, qq.w, a1);
-      }
-      s[g] = valid ? (a0 + a1) * scale_log2 : -INFINITY;
-    }
-
-    // ---- online softmax -------------------------------------------------------
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const float m_new = fmaxf(m[g], wave_max(s[g]));
-      const float alpha = fast_exp2(m[g] - m_new);
-      const float p = fast_exp2(s[g] - m_new);
-      l[g] = l[g] * alpha + p;
-#pragma unroll
-      for (int j = 0; j < VI; ++j) acc[g][j] *= alpha;
-      m[g] = m_new;
-      p_lds[g][lane] = p;
-    }
-    __syncthreads();
-
-    // ---- P.V --------------------------------------------------------------------
-#pragma unroll
-    for (int b = 0; b < BPT; ++b) {
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const float4 pa = *reinterpret_cast<const float4 *>(&p_lds[g][b * BS + part * 8]);
-        const float4 pb = *reinterpret_cast<const float4 *>(&p_lds[g][b * BS + part * 8 + 4]);
-#pragma unroll
-        for (int j = 0; j < VI; ++j) {
-          float a = acc[g][j];
-          a = fma2<T>(vreg[b][j].x, pa.x, pa.y, a);
-          a = fma2<T>(vreg[b][j].y, pa.z, pa.w, a);
-          a = fma2<T>(vreg[b][j].z, pb.x, pb.y, a);
-          a = fma2<T>(vreg[b][j].w, pb.z, pb.w, a);
-          acc[g][j] = a;
-        }
-      }
-    }
-    __syncthreads();
+    uint4 vreg[Geo::BPT][Geo::VI];
+    issue_tile_loads<BS>(kreg, vreg, kpool, vpool, id, tb, u.t1, lane);
+    consume_tile<T, BS, G>(kreg, vreg, q_s, q_lds[wave], p_lds[wave], m, l, acc, I.scale_log2, tb, u.t1, lane);
   }
-
-  // ---- finish: sum the per-part partials, then write output or a partial ---------
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const float L = wave_sum(l[g]);
-    const int hq = hq0 + g;
-    const int64_t prow = (static_cast<int64_t>(seq) * I.Hq + hq) * I.max_splits + split;
-#pragma unroll
-    for (int j = 0; j < VI; ++j) {
-      float a = acc[g][j];
-      if constexpr (PARTS >= 2) a += dpp_mov<0xB1>(a);
-      if constexpr (PARTS >= 4) a += dpp_mov<0x4E>(a);
-      const int d = j * (64 / PARTS) + lane / PARTS;
-      if (part == 0) {
-        if (single) {
-          uint16_t *o = static_cast<uint16_t *>(I.out) + static_cast<int64_t>(seq) * I.out_stride + hq * D;
-          o[d] = to_storage<T>(a / L);
-        } else {
-          I.ws_acc[prow * D + d] = a;
-        }
-      }
-    }
-    if (!single && lane == 0) {
-      I.ws_ml[prow * 2] = m[g];
-      I.ws_ml[prow * 2 + 1] = L;
-    }
-  }
+  stash_wave_partial<BS, G>(m, l, acc, x_acc[wave], x_ml[wave], lane);
+  __syncthreads();
+  if (wave != 0) return;
+  merge_and_write<T, G, NW>(I, u, partition, x_acc, x_ml, lane);
 }
 
-// One block of 128 threads per (sequence, query head) with more than one partition.
-template <typename T>
-__global__ __launch_bounds__(128) void paged_decode_reduce_kernel(const DecodeParams P) {
-  constexpr int D = kHeadSize;
-  const int row = blockIdx.x;
-  int ii = 0;
-#pragma unroll
-  for (int k = 1; k < MUXA_MAX_DECODE_ITEMS; ++k)
-    if (k < P.n_items && row >= P.it[k].row_begin) ii = k;
-  const DecodeItemDev &I = P.it[ii];
-  const int local = row - I.row_begin;
-  const int seq = local / I.Hq;
-  const int hq = local - seq * I.Hq;
-  const int ctx = min(I.ctx[seq], I.max_ctx);
-  if (ctx <= P.partition) return;   // written directly by the main kernel
-  const int n = (ctx + P.partition - 1) / P.partition;
-  const int64_t base = (static_cast<int64_t>(seq) * I.Hq + hq) * I.max_splits;
-  const int d = threadIdx.x;
-  float M = -INFINITY;
-  for (int i = 0; i < n; ++i) M = fmaxf(M, I.ws_ml[(base + i) * 2]);
-  float L = 0.f, a = 0.f;
-  for (int i = 0; i < n; ++i) {
-    const float wgt = fast_exp2(I.ws_ml[(base + i) * 2] - M);
-    L += I.ws_ml[(base + i) * 2 + 1] * wgt;
-    a += I.ws_acc[(base + i) * D + d] * wgt;
-  }
-  uint16_t *o = static_cast<uint16_t *>(I.out) + static_cast<int64_t>(seq) * I.out_stride + hq * D;
-  o[d] = to_storage<T>(a / L);
+// Zero-fills the arrival counters (a kernel rather than a memset node so the
+// call can be captured into a graph).
+__global__ void fill_zero_kernel(int32_t *p, int64_t n) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
 }
 
 // ---------------------------------------------------------------------------
@@ -301,17 +495,38 @@ int pick_group(int ratio) {
   return 1;
 }
 
-struct ItemWs { size_t acc_off, ml_off; int max_splits; };
+struct ItemPlan {
+  size_t counters_off, acc_off, ml_off;
+  int max_splits;
+  int64_t units;      // (sequence, partition) pairs reserved in the direct kernel's grid
+};
 
-// Workspace layout: for every item, acc [B,Hq,max_splits,128] fp32 then ml
-// [B,Hq,max_splits,2] fp32; items whose contexts fit one partition take none.
-size_t plan_workspace(const MuxDecodeItem *items, int n_items, int partition, ItemWs *out) {
-  size_t off = 0;
+// Workspace layout: a FIXED leading region of MUXA_DECODE_COUNTER_BYTES holds
+// the arrival counters (one int32 per sequence and head group, items back to
+// back) so that its position never depends on the shapes of a call and no
+// call's partials can land on another call's counters; then per item acc
+// [B,Hq,max_splits,128] fp32 and ml [B,Hq,max_splits,2] fp32.  Calls whose
+// contexts all fit one partition need no workspace.  Returns total bytes, or
+// SIZE_MAX when the counters do not fit the fixed region.
+size_t plan_workspace(const MuxDecodeItem *items, int n_items, int partition, ItemPlan *out) {
+  size_t counters = 0;
+  size_t off = MUXA_DECODE_COUNTER_BYTES;
+  bool any = false;
   for (int i = 0; i < n_items; ++i) {
-    const int ms = std::max(1, (items[i].max_context_len + partition - 1) / partition);
-    ItemWs w{0, 0, ms};
-    if (ms > 1) {
-      const size_t rows = static_cast<size_t>(items[i].num_seqs) * items[i].num_q_heads * ms;
+    const MuxDecodeItem &it = items[i];
+    ItemPlan w{0, 0, 0, std::max(1, (it.max_context_len + partition - 1) / partition), 0};
+    // Upper bound on the number of pairs: every sequence has at most
+    // max_splits of them, and all sequences together at most
+    // floor(sum ctx / partition) full ones plus one remainder each.
+    w.units = static_cast<int64_t>(it.num_seqs) * w.max_splits;
+    if (it.total_context_len > 0)
+      w.units = std::min<int64_t>(w.units, it.total_context_len / partition + it.num_seqs);
+    if (w.max_splits > 1 && it.num_seqs > 0) {
+      any = true;
+      const int G = pick_group(it.num_q_heads / it.num_kv_heads);
+      w.counters_off = counters;
+      counters += static_cast<size_t>(it.num_seqs) * (it.num_q_heads / G) * sizeof(int32_t);
+      const size_t rows = static_cast<size_t>(it.num_seqs) * it.num_q_heads * w.max_splits;
       w.acc_off = off;
       off += rows * kHeadSize * sizeof(float);
       w.ml_off = off;
@@ -320,19 +535,27 @@ size_t plan_workspace(const MuxDecodeItem *items, int n_items, int partition, It
     }
     if (out) out[i] = w;
   }
+  if (!any) return 0;
+  if (counters > MUXA_DECODE_COUNTER_BYTES) return SIZE_MAX;
   return off;
+}
+
+template <typename T, int BS, int G>
+hipError_t launch_g(const DecodeParams &P, int grid, hipStream_t st) {
+  constexpr int NW = kWavesPerGroup;
+  hipLaunchKernelGGL((paged_decode_kernel<T, BS, G, NW>), dim3(grid), dim3(64 * NW), 0, st, P);
+  return hipGetLastError();
 }
 
 template <typename T, int BS>
 hipError_t launch_main(int G, const DecodeParams &P, int grid, hipStream_t st) {
   switch (G) {
-    case 1: hipLaunchKernelGGL((paged_decode_kernel<T, BS, 1>), dim3(grid), dim3(64), 0, st, P); break;
-    case 2: hipLaunchKernelGGL((paged_decode_kernel<T, BS, 2>), dim3(grid), dim3(64), 0, st, P); break;
-    case 4: hipLaunchKernelGGL((paged_decode_kernel<T, BS, 4>), dim3(grid), dim3(64), 0, st, P); break;
-    case 8: hipLaunchKernelGGL((paged_decode_kernel<T, BS, 8>), dim3(grid), dim3(64), 0, st, P); break;
+    case 1: return launch_g<T, BS, 1>(P, grid, st);
+    case 2: return launch_g<T, BS, 2>(P, grid, st);
+    case 4: return launch_g<T, BS, 4>(P, grid, st);
+    case 8: return launch_g<T, BS, 8>(P, grid, st);
     default: return hipErrorInvalidValue;
   }
-  return hipGetLastError();
 }
 
 template <typename T>
@@ -350,7 +573,7 @@ int32_t validate_item(const MuxDecodeItem &it, int block_size) {
   if (it.num_seqs < 0 || it.num_q_heads <= 0 || it.num_kv_heads <= 0) return MUXA_EINVAL;
   if (it.num_q_heads % it.num_kv_heads != 0) return MUXA_EINVAL;
   if (it.layer < 0 || it.layer >= it.num_layers) return MUXA_EINVAL;
-  if (it.max_blocks < 0 || it.max_context_len < 0) return MUXA_EINVAL;
+  if (it.max_blocks < 0 || it.max_context_len < 0 || it.total_context_len < 0) return MUXA_EINVAL;
   // The grid is sized from max_context_len and every table row must be able
   // to hold that many tokens.
   if (static_cast<int64_t>(it.max_context_len) > static_cast<int64_t>(it.max_blocks) * block_size)
@@ -375,6 +598,19 @@ size_t mux_paged_decode_workspace_bytes(const MuxDecodeItem *items, int32_t n_it
   return mux::plan_workspace(items, n_items, partition, nullptr);
 }
 
+int32_t mux_paged_decode_workspace_init(void *workspace, size_t workspace_bytes, void *stream) {
+  if (!workspace || workspace_bytes == 0) return MUXA_OK;
+  if (reinterpret_cast<uintptr_t>(workspace) & 15u) return MUXA_EINVAL;
+  const int64_t n = static_cast<int64_t>(std::min<size_t>(workspace_bytes, MUXA_DECODE_COUNTER_BYTES) /
+                                        sizeof(int32_t));
+  if (n == 0) return MUXA_OK;
+  hipLaunchKernelGGL(mux::fill_zero_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<int32_t *>(workspace), n);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return mux::hip_fail(e);
+  return MUXA_OK;
+}
+
 int32_t mux_multi_decode(const MuxDecodeItem *items, int32_t n_items,
                          const void *k_pool, const void *v_pool, int64_t num_pool_blocks,
                          int32_t head_size, int32_t block_size, int32_t dtype,
@@ -394,13 +630,15 @@ int32_t mux_multi_decode(const MuxDecodeItem *items, int32_t n_items,
     if (rc != MUXA_OK) return rc;
   }
   const int partition = choose_partition(items, n_items, partition_size);
-  ItemWs ws[MUXA_MAX_DECODE_ITEMS];
-  const size_t need = plan_workspace(items, n_items, partition, ws);
+  ItemPlan plan[MUXA_MAX_DECODE_ITEMS];
+  const size_t need = plan_workspace(items, n_items, partition, plan);
+  if (need == SIZE_MAX) return MUXA_EUNSUPPORTED;   // more (sequence, head group) pairs than counters
   if (need > 0 && (!workspace || workspace_bytes < need)) return MUXA_EWORKSPACE;
   if (need > 0 && (reinterpret_cast<uintptr_t>(workspace) & 15u)) return MUXA_EINVAL;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  char *ws = static_cast<char *>(workspace);
 
-  // Items are launched in groups that share G (query heads per wave).
+  // Items are launched in groups that share G (query heads per workgroup).
   bool done[MUXA_MAX_DECODE_ITEMS] = {false};
   for (int first = 0; first < n_items; ++first) {
     if (done[first]) continue;
@@ -411,14 +649,14 @@ int32_t mux_multi_decode(const MuxDecodeItem *items, int32_t n_items,
     P.partition = partition;
     P.last_block = static_cast<int32_t>(std::min<int64_t>(num_pool_blocks - 1, 0x7fffffff));
     P.n_items = 0;
-    int64_t work = 0, rows = 0;
-    bool any_split = false;
+    int64_t work = 0;
     for (int i = first; i < n_items; ++i) {
       if (done[i]) continue;
       const MuxDecodeItem &it = items[i];
       if (pick_group(it.num_q_heads / it.num_kv_heads) != G) continue;
       done[i] = true;
       if (it.num_seqs == 0 || it.max_context_len == 0) continue;
+      const bool split = plan[i].max_splits > 1;
       DecodeItemDev &d = P.it[P.n_items++];
       d.out = it.out;
       d.q = it.q;
@@ -427,37 +665,26 @@ int32_t mux_multi_decode(const MuxDecodeItem *items, int32_t n_items,
       d.tables = it.block_tables +
                  static_cast<int64_t>(it.layer) * it.num_seqs * it.num_kv_heads * it.max_blocks;
       d.ctx = it.context_lens;
-      d.ws_acc = ws[i].max_splits > 1
-                     ? reinterpret_cast<float *>(static_cast<char *>(workspace) + ws[i].acc_off) : nullptr;
-      d.ws_ml = ws[i].max_splits > 1
-                    ? reinterpret_cast<float *>(static_cast<char *>(workspace) + ws[i].ml_off) : nullptr;
+      d.ws_acc = split ? reinterpret_cast<float *>(ws + plan[i].acc_off) : nullptr;
+      d.ws_ml = split ? reinterpret_cast<float *>(ws + plan[i].ml_off) : nullptr;
+      d.counters = split ? reinterpret_cast<int32_t *>(ws + plan[i].counters_off) : nullptr;
       d.B = it.num_seqs;
       d.Hq = it.num_q_heads;
       d.Hkv = it.num_kv_heads;
       d.ratio = it.num_q_heads / it.num_kv_heads;
       d.max_blocks = it.max_blocks;
-      d.max_splits = ws[i].max_splits;
+      d.max_splits = plan[i].max_splits;
       d.max_ctx = it.max_context_len;
       d.work_begin = static_cast<int32_t>(work);
-      d.row_begin = static_cast<int32_t>(rows);
       d.scale_log2 = it.scale * 1.4426950408889634f;
-      work += static_cast<int64_t>(it.num_seqs) * (it.num_q_heads / G) * ws[i].max_splits;
-      rows += static_cast<int64_t>(it.num_seqs) * it.num_q_heads;
-      any_split = any_split || ws[i].max_splits > 1;
-      if (work > 0x7fffffff || rows > 0x7fffffff) return MUXA_EUNSUPPORTED;
+      work += plan[i].units * (it.num_q_heads / G);
+      if (work > 0x7fffffff) return MUXA_EUNSUPPORTED;
     }
     if (P.n_items == 0) continue;
-    hipError_t e = dtype == MUXA_DTYPE_F16 ? launch_bs<F16>(block_size, G, P, static_cast<int>(work), st)
-                                           : launch_bs<BF16>(block_size, G, P, static_cast<int>(work), st);
+    const int grid = static_cast<int>(work);
+    hipError_t e = dtype == MUXA_DTYPE_F16 ? launch_bs<F16>(block_size, G, P, grid, st)
+                                           : launch_bs<BF16>(block_size, G, P, grid, st);
     if (e != hipSuccess) return hip_fail(e);
-    if (any_split) {
-      if (dtype == MUXA_DTYPE_F16)
-        hipLaunchKernelGGL((paged_decode_reduce_kernel<F16>), dim3(static_cast<int>(rows)), dim3(128), 0, st, P);
-      else
-        hipLaunchKernelGGL((paged_decode_reduce_kernel<BF16>), dim3(static_cast<int>(rows)), dim3(128), 0, st, P);
-      e = hipGetLastError();
-      if (e != hipSuccess) return hip_fail(e);
-    }
   }
   return MUXA_OK;
 }
@@ -477,6 +704,7 @@ int32_t mux_paged_decode(void *out, int64_t out_row_stride, const void *q, int64
   it.q_row_stride = q_row_stride;
   it.block_tables = block_tables;
   it.context_lens = context_lens;
+  it.total_context_len = 0;
   it.layer = layer;
   it.num_layers = num_layers;
   it.num_seqs = num_seqs;

@@ -97,6 +97,7 @@ class DecodeCall:
     max_context_len: int
     scale: float
     layer: int = 0
+    total_context_len: int = 0    # host-side bound on sum(context_lens); 0 = unknown
 
     def to_item(self) -> _lib.MuxDecodeItem:
         bt, cl = self.block_tables, self.context_lens
@@ -120,6 +121,7 @@ class DecodeCall:
         it.num_q_heads, it.num_kv_heads = self.q.shape[1] // HEAD_SIZE, Hkv
         it.max_blocks, it.max_context_len = max_blocks, int(self.max_context_len)
         it.scale = float(self.scale)
+        it.total_context_len = int(self.total_context_len)
         return it
 
 
@@ -127,13 +129,14 @@ _workspaces = {}
 
 
 def _workspace(nbytes: int, device) -> Optional[torch.Tensor]:
-    """Grow-only scratch for split partials, one per (device, stream)."""
+    """Grow-only scratch for split partials, one per (device, stream).  Born
+    zeroed: it starts with arrival counters that every launch leaves at zero."""
     if nbytes == 0:
         return None
     key = (device, torch.cuda.current_stream(device).cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 
@@ -160,8 +163,10 @@ def multi_decode(calls: List[DecodeCall], k_pool: torch.Tensor, v_pool: torch.Te
 
 
 def paged_decode(out, q, k_pool, v_pool, block_tables, context_lens, max_context_len, scale,
-                 layer: int = 0, partition_size: int = 0, workspace=None, stream=None) -> None:
-    multi_decode([DecodeCall(out, q, block_tables, context_lens, max_context_len, scale, layer)],
+                 layer: int = 0, partition_size: int = 0, workspace=None, stream=None,
+                 total_context_len: int = 0) -> None:
+    multi_decode([DecodeCall(out, q, block_tables, context_lens, max_context_len, scale, layer,
+                             total_context_len)],
                  k_pool, v_pool, partition_size, workspace, stream)
 
 

@@ -27,7 +27,7 @@ def _nan_pool(n, bs, dtype):
 
 
 def _decode_case(seed, ctx_lens, Hq, Hkv, bs, dtype=torch.float16, partition=0, num_layers=1, layer=0,
-                 q_in_qkv=False, extra_blocks=7):
+                 q_in_qkv=False, extra_blocks=7, hint=False, repeat=1):
     """Builds pool + tables on the host with the oracle's cache write, runs the
     GPU decode, returns (gpu_out fp32, oracle_out fp32)."""
     rng = np.random.Generator(np.random.PCG64(seed))
@@ -62,9 +62,11 @@ def _decode_case(seed, ctx_lens, Hq, Hkv, bs, dtype=torch.float16, partition=0, 
 
     dq = (qkv.to(DEV)[:, :Hq * HEAD_SIZE]) if q_in_qkv else q.to(DEV)
     out = torch.full((pad, Hq * HEAD_SIZE), 7.0, dtype=dtype, device=DEV)
-    ops.paged_decode(out, dq, k_pool.to(DEV), v_pool.to(DEV), torch.from_numpy(bt).to(DEV),
-                     torch.from_numpy(ctx).to(DEV), int(ctx.max()), scale, layer=layer,
-                     partition_size=partition)
+    dkp, dvp, dbt, dctx = k_pool.to(DEV), v_pool.to(DEV), torch.from_numpy(bt).to(DEV), torch.from_numpy(ctx).to(DEV)
+    for _ in range(repeat):     # repeated launches reuse the workspace (arrival counters must self-reset)
+        out.fill_(7.0)
+        ops.paged_decode(out, dq, dkp, dvp, dbt, dctx, int(ctx.max()), scale, layer=layer,
+                         partition_size=partition, total_context_len=int(ctx.sum()) if hint else 0)
     torch.cuda.synchronize()
     got = out.float().cpu()
     assert (got[B:] == 7.0).all(), "padding rows of out must not be written"
@@ -169,6 +171,19 @@ def test_decode_split_context_equals_single_pass(partition):
     _announce(f"decode split partition={partition}")
     ctx = [1, 64, 65, 200, 513, 777, 1024, 1500]
     got, want = _decode_case(3, ctx, 3, 3, 16, partition=partition)
+    _check(got, want)
+
+
+@pytest.mark.parametrize("B", [65, 130])
+@pytest.mark.parametrize("hint", [False, True])
+def test_decode_more_sequences_than_a_wave(B, hint):
+    """Unit enumeration walks the context lengths 64 sequences at a time."""
+    _announce(f"decode B={B} hint={hint}")
+    rng = np.random.Generator(np.random.PCG64(B))
+    ctx = rng.integers(1, 400, size=B)
+    ctx[::7] = 128          # exact multiples of the partition: no remainder unit
+    ctx[3] = 1
+    got, want = _decode_case(7, ctx, 2, 2, 16, partition=128, hint=hint, repeat=3)
     _check(got, want)
 
 
@@ -279,9 +294,11 @@ def test_decode_config2_full_size_pool():
     workloads.fill_blocks(dk, dv, used, seed=0)
     for i, m in enumerate(models):
         m.to_device(DEV, torch.float16, seed=20 + i)
-    calls = [ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale)
+    calls = [ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                            total_context_len=int(m.context_lens.sum()))
              for m in models]
-    ops.multi_decode(calls, dk, dv)
+    for _ in range(3):
+        ops.multi_decode(calls, dk, dv)
     torch.cuda.synchronize()
     ks, vs, tables = workloads.compact_to_host(dk, dv, models, bs)
     del dk, dv
