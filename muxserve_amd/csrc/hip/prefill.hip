@@ -1,8 +1,306 @@
-// Causal prefill attention (placeholder until the MFMA kernel lands).
+// Causal prefill attention on the fresh q, k, v of a batch of packed prompts,
+// gfx950 MFMA (v_mfma_f32_32x32x16_{f16,bf16}).
+//
+// One workgroup = 128 query rows of one head of one prompt, 4 waves x 32 rows.
+// Keys/values stream through LDS in tiles of 64 tokens shared by the 4 waves.
+// Each wave keeps the TRANSPOSED problem so that probabilities never leave
+// registers:
+//     S^T[key][q] = K . Q^T      A = K tile   (LDS, row-major, 16-byte frags)
+//                                B = Q^T      (registers, loaded once)
+//     O^T[d][q]  += V^T . P^T    A = V^T tile (LDS, stored transposed)
+//                                B = P^T      = the S^T accumulators, converted
+// In the 32x32 accumulator layout a lane owns ONE query column (q = lane%32)
+// and 16 of the 32 keys of a block, so softmax statistics are per-lane scalars
+// (one exchange with lane^32), the rescale of O^T is a per-lane multiply, and
+// the accumulator registers of S^T are, in order, exactly the 8-element
+// B-operand fragments of the P.V products - provided the V^T fragments use the
+// same key order (two groups of four keys), which costs nothing because V^T is
+// read from LDS anyway.
+// V is transposed on its way into LDS: a thread loads 4 keys x 8 dims, does the
+// 4x8 16-bit transpose with byte permutes, and writes 8 rows of V^T.
+// The next tile's global loads are issued before the current tile's math.
 #include "mux_common.h"
 
-extern "C" int32_t mux_prefill_causal(void *, int64_t, const void *, int64_t, const void *, const void *,
-                                      int64_t, const int32_t *, int32_t, int32_t, int32_t, int32_t,
-                                      int32_t, float, int32_t, void *) {
-  return MUXA_EUNSUPPORTED;
+namespace mux {
+
+typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf16 __attribute__((ext_vector_type(8)));
+typedef float v16f32 __attribute__((ext_vector_type(16)));
+
+constexpr int kBM = 128;                 // query rows per workgroup
+constexpr int kBN = 64;                  // keys per tile
+constexpr int kKRow = kHeadSize + 8;     // K tile row length in elements (272 B: 16-byte frags, rows 4 banks apart)
+constexpr int kVRow = kBN + 8;           // V^T tile row length in elements (144 B)
+
+union Frag {
+  uint4 u;
+  v8f16 h;
+  v8bf16 b;
+};
+
+template <typename T>
+__device__ __forceinline__ v16f32 mfma(const Frag &a, const Frag &b, v16f32 c) {
+  if constexpr (__is_same(T, F16)) return __builtin_amdgcn_mfma_f32_32x32x16_f16(a.h, b.h, c, 0, 0, 0);
+  else return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.b, b.b, c, 0, 0, 0);
+}
+
+// Two fp32 -> one packed pair in storage type T.
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  return static_cast<uint32_t>(to_storage<T>(lo)) | (static_cast<uint32_t>(to_storage<T>(hi)) << 16);
+}
+
+struct PrefillParams {
+  uint16_t *out;
+  const uint16_t *q, *k, *v;
+  int64_t out_stride, q_stride, kv_stride;
+  const int32_t *cu_seqlens;
+  int32_t ratio;          // query heads per kv head
+  int32_t q_tiles;        // grid.x
+  float scale_log2;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void prefill_causal_kernel(const PrefillParams P) {
+  constexpr int D = kHeadSize;
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[kBN * kKRow];
+  __shared__ __attribute__((aligned(16))) uint16_t Vt[D * kVRow];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int hq = blockIdx.y;
+  const int hk = hq / P.ratio;
+  const int prompt = blockIdx.z;
+  const int seq_begin = P.cu_seqlens[prompt];
+  const int len = P.cu_seqlens[prompt + 1] - seq_begin;
+  // Heaviest tiles (most keys) first.
+  const int q0 = (P.q_tiles - 1 - static_cast<int>(blockIdx.x)) * kBM;
+  if (q0 >= len) return;
+
+  const int qcol = lane & 31;            // this lane's query column / fragment row
+  const int half = lane >> 5;            // which 8 of a fragment's 16 k-slots
+  const int wq0 = q0 + wave * 32;        // first query row of this wave
+  const int my_q = wq0 + qcol;           // this lane's query position inside the prompt
+
+  // ---- Q^T fragments: Q[my_q][16 s + 8 half .. +7], s = 0..7 ------------------------
+  Frag qf[8];
+  {
+    const bool ok = my_q < len;
+    const uint16_t *qp = P.q + static_cast<int64_t>(seq_begin + (ok ? my_q : 0)) * P.q_stride + hq * D + 8 * half;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) qf[s].u = ok ? *reinterpret_cast<const uint4 *>(qp + 16 * s) : make_uint4(0, 0, 0, 0);
+  }
+
+  v16f32 oacc[4];                        // O^T[d = 32 mb + ...][q]
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) oacc[mb][i] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  // Keys needed by this workgroup: positions 0 .. min(len, q0 + 128) - 1.
+  const int kv_end = min(len, q0 + kBM);
+  const int n_tiles = (kv_end + kBN - 1) / kBN;
+
+  // Global -> register staging of one K/V tile.  K: thread takes chunk
+  // (key = tid/16 + 16 i, dchunk = tid%16).  V: thread takes keys 4 kg .. 4 kg+3
+  // (kg = tid%16) of dchunk vc = tid/16.
+  const int kc = tid & 15, kk = tid >> 4;
+  const int vg = tid & 15, vc = tid >> 4;
+  uint4 kst[4], vst[4];
+  auto load_tile = [&](int t) {
+    const int k0 = t * kBN;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = k0 + kk + 16 * i;
+      kst[i] = key < len ? *reinterpret_cast<const uint4 *>(
+                               P.k + static_cast<int64_t>(seq_begin + key) * P.kv_stride + hk * D + 8 * kc)
+                         : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = k0 + 4 * vg + i;
+      // Rows past the prompt are zero so that 0 * garbage cannot make a NaN.
+      vst[i] = key < len ? *reinterpret_cast<const uint4 *>(
+                               P.v + static_cast<int64_t>(seq_begin + key) * P.kv_stride + hk * D + 8 * vc)
+                         : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<uint4 *>(&Ks[(kk + 16 * i) * kKRow + 8 * kc]) = kst[i];
+    // 4 keys x 8 dims -> 8 rows of V^T, 4 keys (8 bytes) each.
+    const uint32_t a[4][4] = {{vst[0].x, vst[0].y, vst[0].z, vst[0].w},
+                              {vst[1].x, vst[1].y, vst[1].z, vst[1].w},
+                              {vst[2].x, vst[2].y, vst[2].z, vst[2].w},
+                              {vst[3].x, vst[3].y, vst[3].z, vst[3].w}};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {        // dword w of a chunk holds dims 2w, 2w+1
+      // low halves -> dim 2w, high halves -> dim 2w+1
+      const uint32_t lo01 = __builtin_amdgcn_perm(a[1][w], a[0][w], 0x05040100u);
+      const uint32_t lo23 = __builtin_amdgcn_perm(a[3][w], a[2][w], 0x05040100u);
+      const uint32_t hi01 = __builtin_amdgcn_perm(a[1][w], a[0][w], 0x07060302u);
+      const uint32_t hi23 = __builtin_amdgcn_perm(a[3][w], a[2][w], 0x07060302u);
+      *reinterpret_cast<uint2 *>(&Vt[(8 * vc + 2 * w) * kVRow + 4 * vg]) = make_uint2(lo01, lo23);
+      *reinterpret_cast<uint2 *>(&Vt[(8 * vc + 2 * w + 1) * kVRow + 4 * vg]) = make_uint2(hi01, hi23);
+    }
+  };
+
+  load_tile(0);
+  for (int t = 0; t < n_tiles; ++t) {
+    const int k0 = t * kBN;
+    __syncthreads();                     // everyone is done reading the previous tile
+    store_tile();
+    __syncthreads();
+    if (t + 1 < n_tiles) load_tile(t + 1);
+    if (k0 > wq0 + 31) continue;         // every key of the tile is in this wave's future
+
+    // ---- S^T = K . Q^T : two 32-key blocks ------------------------------------------
+    v16f32 sacc[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        Frag kf;
+        kf.u = *reinterpret_cast<const uint4 *>(&Ks[(32 * kb + qcol) * kKRow + 16 * s + 8 * half]);
+        sacc[kb] = mfma<T>(kf, qf[s], sacc[kb]);
+      }
+    }
+
+    // ---- softmax over keys, per query column --------------------------------------
+    // register i of block kb is key k0 + 32 kb + 8 (i/4) + 4 half + i%4
+    float mx = -INFINITY;
+    const bool diag = k0 + kBN - 1 > wq0;   // some (key, q) pair of this wave's tile is masked
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float sv = sacc[kb][i] * P.scale_log2;
+        if (diag) {
+          const int key = k0 + 32 * kb + 8 * (i / 4) + 4 * half + (i % 4);
+          if (key > my_q) sv = -INFINITY;
+        }
+        sacc[kb][i] = sv;
+        mx = fmaxf(mx, sv);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    // Rows past the prompt may have no valid key at all; keep them finite.
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = fast_exp2(m_run - m_use);
+    float psum = 0.f;
+    Frag pf[4];                          // B fragments: [kb][step] -> index 2 kb + st
+    // bf16 keeps only 8 mantissa bits of a probability, which alone would cost
+    // more than the 2e-3 budget, so bf16 P is carried as hi + lo parts.
+    constexpr bool kSplitP = __is_same(T, BF16);
+    Frag pf_lo[kSplitP ? 4 : 1];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      float p[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        p[i] = fast_exp2(sacc[kb][i] - m_use);
+        psum += p[i];
+      }
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        pf[2 * kb + st].u = make_uint4(pack2<T>(p[8 * st + 0], p[8 * st + 1]), pack2<T>(p[8 * st + 2], p[8 * st + 3]),
+                                       pack2<T>(p[8 * st + 4], p[8 * st + 5]), pack2<T>(p[8 * st + 6], p[8 * st + 7]));
+        if constexpr (kSplitP) {
+          float r[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            r[j] = p[8 * st + j] - __uint_as_float(static_cast<uint32_t>(f32_to_bf16_bits(p[8 * st + j])) << 16);
+          pf_lo[2 * kb + st].u = make_uint4(pack2<T>(r[0], r[1]), pack2<T>(r[2], r[3]),
+                                            pack2<T>(r[4], r[5]), pack2<T>(r[6], r[7]));
+        }
+      }
+    }
+    l_run = l_run * alpha + psum;
+    m_run = m_use;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[mb][i] *= alpha;
+
+    // ---- O^T += V^T . P^T ---------------------------------------------------------------
+    // k-slot j of lane half h in step (kb, st) is key 32 kb + 16 st + 8 (j/4) + 4 h + j%4
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const uint16_t *vr = &Vt[(32 * mb + qcol) * kVRow + 16 * ks + 4 * half];
+        const uint2 lo = *reinterpret_cast<const uint2 *>(vr);
+        const uint2 hi = *reinterpret_cast<const uint2 *>(vr + 8);
+        Frag vf;
+        vf.u = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        oacc[mb] = mfma<T>(vf, pf[ks], oacc[mb]);
+        if constexpr (kSplitP) oacc[mb] = mfma<T>(vf, pf_lo[ks], oacc[mb]);
+      }
+    }
+  }
+
+  // ---- normalise and store: register i of block mb is d = 32 mb + 8 (i/4) + 4 half + i%4 ------
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  if (my_q < len) {
+    const float inv = 1.f / l_tot;
+    uint16_t *op = P.out + static_cast<int64_t>(seq_begin + my_q) * P.out_stride + hq * D + 4 * half;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const uint2 w2 = make_uint2(pack2<T>(oacc[mb][4 * g] * inv, oacc[mb][4 * g + 1] * inv),
+                                    pack2<T>(oacc[mb][4 * g + 2] * inv, oacc[mb][4 * g + 3] * inv));
+        *reinterpret_cast<uint2 *>(op + 32 * mb + 8 * g) = w2;
+      }
+  }
+}
+
+}  // namespace mux
+
+extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const void *q, int64_t q_row_stride,
+                                      const void *k, const void *v, int64_t kv_row_stride,
+                                      const int32_t *cu_seqlens, int32_t num_prompts, int32_t max_prompt_len,
+                                      int32_t num_q_heads, int32_t num_kv_heads, int32_t head_size,
+                                      float scale, int32_t dtype, void *stream) {
+  using namespace mux;
+  if (!out || !q || !k || !v || !cu_seqlens) return MUXA_EINVAL;
+  if (num_prompts < 0 || max_prompt_len < 0 || num_q_heads <= 0 || num_kv_heads <= 0) return MUXA_EINVAL;
+  if (num_q_heads % num_kv_heads != 0) return MUXA_EINVAL;
+  if (head_size != kHeadSize) return MUXA_EUNSUPPORTED;
+  if (dtype != MUXA_DTYPE_F16 && dtype != MUXA_DTYPE_BF16) return MUXA_EUNSUPPORTED;
+  if (q_row_stride < static_cast<int64_t>(num_q_heads) * kHeadSize ||
+      out_row_stride < static_cast<int64_t>(num_q_heads) * kHeadSize ||
+      kv_row_stride < static_cast<int64_t>(num_kv_heads) * kHeadSize)
+    return MUXA_EINVAL;
+  // 16-byte fragment loads and 8-byte output stores.
+  if (q_row_stride % 8 || kv_row_stride % 8 || out_row_stride % 4) return MUXA_EINVAL;
+  const uintptr_t a16 = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v);
+  if ((a16 & 15u) || (reinterpret_cast<uintptr_t>(out) & 7u)) return MUXA_EINVAL;
+  if (num_q_heads > 65535 || num_prompts > 65535) return MUXA_EUNSUPPORTED;
+  if (num_prompts == 0 || max_prompt_len == 0) return MUXA_OK;
+
+  PrefillParams P;
+  P.out = static_cast<uint16_t *>(out);
+  P.q = static_cast<const uint16_t *>(q);
+  P.k = static_cast<const uint16_t *>(k);
+  P.v = static_cast<const uint16_t *>(v);
+  P.out_stride = out_row_stride;
+  P.q_stride = q_row_stride;
+  P.kv_stride = kv_row_stride;
+  P.cu_seqlens = cu_seqlens;
+  P.ratio = num_q_heads / num_kv_heads;
+  P.q_tiles = (max_prompt_len + kBM - 1) / kBM;
+  P.scale_log2 = scale * 1.4426950408889634f;
+  const dim3 grid(P.q_tiles, num_q_heads, num_prompts);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == MUXA_DTYPE_F16) hipLaunchKernelGGL(prefill_causal_kernel<F16>, grid, dim3(256), 0, st, P);
+  else hipLaunchKernelGGL(prefill_causal_kernel<BF16>, grid, dim3(256), 0, st, P);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(e);
+  return MUXA_OK;
 }

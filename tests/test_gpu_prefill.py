@@ -1,0 +1,149 @@
+"""GPU parity: causal prefill attention (MFMA) against the CPU oracle
+(<= 2e-3 max-abs, fp16/bf16 in, fp32 accumulate), then the prefill-shaped cache
+write into head-wise slot mappings, bit-exact.  All through the C ABI.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import attn_oracle as orc
+from muxserve_amd import ops, workloads
+from muxserve_amd.pool import HEAD_SIZE, allocate_gpu_cache
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 2e-3
+D = HEAD_SIZE
+
+
+def _announce(msg):
+    print(f"[case] {msg}", flush=True)
+
+
+def _bound(want, dtype):
+    b = torch.full_like(want, TOL)
+    if dtype == torch.bfloat16:      # + rounding of the result to bf16 (8-bit mantissa)
+        b = b + want.abs() * 2.0 ** -8
+    return b
+
+
+def _run_prefill(seed, lens, Hq, Hkv, dtype, in_qkv=True):
+    g = torch.Generator().manual_seed(seed)
+    T = int(sum(lens))
+    pad = (T + 7) // 8 * 8
+    if in_qkv:
+        qkv = torch.randn((pad, (Hq + 2 * Hkv) * D), generator=g).to(dtype)
+        q, k, v = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)     # models/llama.py:157-158
+        dqkv = qkv.to(DEV)
+        dq, dk, dv = dqkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+    else:
+        q = torch.randn((pad, Hq * D), generator=g).to(dtype)
+        k = torch.randn((pad, Hkv * D), generator=g).to(dtype)
+        v = torch.randn((pad, Hkv * D), generator=g).to(dtype)
+        dq, dk, dv = q.to(DEV), k.to(DEV), v.to(DEV)
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32, device=DEV)
+    out = torch.full((pad, Hq * D), 7.0, dtype=dtype, device=DEV)
+    ops.prefill_causal(out, dq, dk, dv, cu, int(max(lens)), D ** -0.5, Hkv)
+    torch.cuda.synchronize()
+    got = out.float().cpu()
+    assert (got[T:] == 7.0).all(), "padding rows must not be written"
+    return got[:T], q, k, v
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv", [(3, 3), (4, 2), (8, 1)])
+def test_prefill_matches_oracle_ragged_prompts(Hq, Hkv, dtype):
+    _announce(f"prefill ragged Hq={Hq} Hkv={Hkv} {dtype}")
+    lens = [1, 7, 64, 33, 128, 129, 300, 31]
+    got, q, k, v = _run_prefill(1, lens, Hq, Hkv, dtype)
+    want = orc.prefill_causal(q, k, v, lens, D ** -0.5, Hkv)
+    assert torch.isfinite(got).all()
+    excess = ((got - want).abs() - _bound(want, dtype)).max().item()
+    assert excess <= 0, f"max-abs error {(got - want).abs().max().item():.3e}"
+
+
+def test_prefill_long_prompt_and_unstrided_inputs():
+    _announce("prefill long prompt")
+    lens = [2048, 5, 700]
+    got, q, k, v = _run_prefill(2, lens, 2, 2, torch.float16, in_qkv=False)
+    want = orc.prefill_causal(q, k, v, lens, D ** -0.5, 2)
+    assert torch.isfinite(got).all()
+    assert (got - want).abs().max().item() <= TOL
+
+
+def test_prefill_first_token_and_block_diagonal_properties():
+    """Row 0 of every prompt equals its own v; changing one prompt's k leaves
+    every other prompt's output bit-identical."""
+    _announce("prefill properties")
+    lens = [40, 130, 9]
+    g = torch.Generator().manual_seed(3)
+    T = sum(lens)
+    q = torch.randn((T, 2 * D), generator=g).half().to(DEV)
+    k = torch.randn((T, 2 * D), generator=g).half().to(DEV)
+    v = torch.randn((T, 2 * D), generator=g).half().to(DEV)
+    cu = torch.tensor([0, 40, 170, 179], dtype=torch.int32, device=DEV)
+    out = torch.zeros_like(q)
+    ops.prefill_causal(out, q, k, v, cu, 130, D ** -0.5, 2)
+    k2 = k.clone()
+    k2[40:170] += 1
+    out2 = torch.zeros_like(q)
+    ops.prefill_causal(out2, q, k2, v, cu, 130, D ** -0.5, 2)
+    torch.cuda.synchronize()
+    for s in (0, 40, 170):
+        assert torch.equal(out[s], v[s])
+    assert torch.equal(out[:40], out2[:40]) and torch.equal(out[170:], out2[170:])
+    assert not torch.equal(out[40:170], out2[40:170])
+
+
+def test_config3_prefill_then_cache_write_bit_exact():
+    """Three shapes, 16 prompts each, lengths lognormal(200, 1.0) in [8, 2048]:
+    attention checked on a subset of heads (the CPU oracle is O(n^2) per head),
+    the cache scatter into seeded random head-wise slot mappings checked
+    bit-exact over the whole pool."""
+    _announce("config 3")
+    bs = 16
+    models = workloads.config3(seed=0)
+    total_blocks = sum(int(((m.prompt_lens + bs - 1) // bs).sum()) * m.num_kv_heads for m in models)
+    N = total_blocks + 1000
+    rng = np.random.Generator(np.random.PCG64(0))
+    ids = rng.permutation(N)
+    dk_pool, dv_pool = allocate_gpu_cache(N, bs, DEV)
+    dk_pool.zero_()
+    dv_pool.zero_()
+    hk_pool, hv_pool = dk_pool.cpu(), dv_pool.cpu()
+    cur = 0
+    for mi, m in enumerate(models):
+        _announce(f"config 3 model {m.name} tokens={m.num_tokens}")
+        g = torch.Generator().manual_seed(10 + mi)
+        Hq, Hkv, T = m.num_q_heads, m.num_kv_heads, m.num_tokens
+        pad = (T + 7) // 8 * 8
+        qkv = torch.randn((pad, (Hq + 2 * Hkv) * D), generator=g).half()
+        dqkv = qkv.to(DEV)
+        dq, dk, dv = dqkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+        q, k, v = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+        cu = torch.from_numpy(m.cu_seqlens()).to(DEV)
+        out = torch.zeros((pad, Hq * D), dtype=torch.float16, device=DEV)
+        ops.prefill_causal(out, dq, dk, dv, cu, int(m.prompt_lens.max()), m.scale, Hkv)
+        slots, used = workloads.prefill_slot_mapping(m.prompt_lens, Hkv, bs, ids[cur:])
+        cur += used
+        ops.reshape_and_cache(dk, dv, dk_pool, dv_pool, torch.from_numpy(slots).to(DEV), num_tokens=T)
+        torch.cuda.synchronize()
+        orc.reshape_and_cache(k, v, hk_pool, hv_pool, torch.from_numpy(slots), num_tokens=T)
+        heads = sorted({0, Hq // 2, Hq - 1})
+        sel = torch.cat([torch.arange(h * D, (h + 1) * D) for h in heads])
+        want = orc.prefill_causal(q[:, sel], k[:, sel], v[:, sel], m.prompt_lens, m.scale, len(heads))
+        got = out[:T].cpu()[:, sel].float()
+        assert torch.isfinite(out[:T]).all()
+        err = (got - want).abs().max().item()
+        assert err <= TOL, f"{m.name}: prefill max-abs error {err:.3e}"
+    assert torch.equal(dk_pool.cpu().view(torch.int16), hk_pool.view(torch.int16))
+    assert torch.equal(dv_pool.cpu().view(torch.int16), hv_pool.view(torch.int16))
+
+
+def test_prefill_rejects_bad_arguments():
+    q = torch.zeros((8, 256), dtype=torch.float16, device=DEV)
+    cu = torch.tensor([0, 8], dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError):
+        ops.prefill_causal(q, q, q[:, :128], q, cu, 8, 1.0, 1)      # k/v shape mismatch
+    with pytest.raises(RuntimeError):
+        ops.prefill_causal(q.cpu(), q.cpu(), q.cpu(), q.cpu(), cu, 8, 1.0, 2)
