@@ -157,6 +157,19 @@ int32_t mux_prefill_causal(void *out, int64_t out_row_stride,
                            int32_t num_q_heads, int32_t num_kv_heads, int32_t head_size,
                            float scale, int32_t dtype, void *stream);
 
+/* ---- Rotary position embedding --------------------------------------------
+ * The attention layer of the reference is PagedAttentionWithRoPE constructed
+ * with rotary_dim = head_dim and base = rope_theta
+ * (muxserve/flexserver/models/llama.py:138-147): NeoX-style rotation of q and k
+ * in place, before the cache write.  positions: int64 [>= num_tokens]
+ * (llm_runtime.py:325).  cos_sin: DEVICE fp32 [max_position, rotary_dim], row p
+ * = [cos(p*f_0..f_{r/2-1}) | sin(...)], f_i = base^(-2i/rotary_dim).  fp32
+ * arithmetic, one rounding to the storage type. */
+int32_t mux_rotary_neox(const int64_t *positions, void *q, int64_t q_row_stride, void *k,
+                        int64_t k_row_stride, const float *cos_sin, int32_t max_position,
+                        int32_t rotary_dim, int32_t num_tokens, int32_t num_q_heads,
+                        int32_t num_kv_heads, int32_t head_size, int32_t dtype, void *stream);
+
 /* ---- CU-masked streams ---------------------------------------------------
  * Replacement for the reference's per-process MPS share
  * (CUDA_MPS_ACTIVE_THREAD_PERCENTAGE, muxserve/muxsched/launcher.py:54-61):

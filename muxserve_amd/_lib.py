@@ -125,6 +125,8 @@ ATTN_SIGNATURES = {
                                  c_f32, c_i32, c_i32, c_vp, c_sz, c_vp]),
     "mux_prefill_causal": (c_i32, [c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i32, c_i32,
                                    c_i32, c_i32, c_i32, c_f32, c_i32, c_vp]),
+    "mux_rotary_neox": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32,
+                                c_i32, c_vp]),
     "mux_stream_create_cu_range": (c_i32, [c_vp, c_i32, c_i32, c_vp]),
     "mux_stream_destroy": (c_i32, [c_vp]),
     "mux_device_cu_info": (c_i32, [c_vp]),

@@ -188,3 +188,56 @@ def prefill_causal(out, q, k, v, cu_seqlens: torch.Tensor, max_prompt_len: int, 
         cu_seqlens.data_ptr(), cu_seqlens.shape[0] - 1, int(max_prompt_len), q.shape[1] // HEAD_SIZE,
         int(num_kv_heads), HEAD_SIZE, float(scale), _dtype_code(q), _stream_ptr(stream))
     _lib.check_attn(rc, "mux_prefill_causal")
+
+
+def rotary_neox(positions: torch.Tensor, q: torch.Tensor, k: torch.Tensor, cos_sin: torch.Tensor,
+                num_tokens: Optional[int] = None, stream=None) -> None:
+    """NeoX rotary embedding in place on q [T_pad, Hq*128] and k [T_pad, Hkv*128];
+    positions int64 [T_pad]; cos_sin fp32 [max_position, rotary_dim] on the device."""
+    _need_cuda(positions, q, k, cos_sin)
+    if positions.dtype != torch.int64 or positions.dim() != 1 or not positions.is_contiguous():
+        raise ValueError("positions: expected contiguous int64 [T]")
+    if cos_sin.dtype != torch.float32 or cos_sin.dim() != 2 or not cos_sin.is_contiguous():
+        raise ValueError("cos_sin: expected contiguous float32 [max_position, rotary_dim]")
+    if q.dtype != k.dtype or q.shape[1] % HEAD_SIZE or k.shape[1] % HEAD_SIZE:
+        raise ValueError("q [T, Hq*128], k [T, Hkv*128] of one dtype expected")
+    T = positions.shape[0] if num_tokens is None else int(num_tokens)
+    if min(q.shape[0], k.shape[0], positions.shape[0]) < T:
+        raise ValueError("fewer rows than tokens")
+    rc = _lib.attn().mux_rotary_neox(positions.data_ptr(), q.data_ptr(), _rows(q, "q"), k.data_ptr(), _rows(k, "k"),
+                                     cos_sin.data_ptr(), cos_sin.shape[0], cos_sin.shape[1], T,
+                                     q.shape[1] // HEAD_SIZE, k.shape[1] // HEAD_SIZE, HEAD_SIZE, _dtype_code(q),
+                                     _stream_ptr(stream))
+    _lib.check_attn(rc, "mux_rotary_neox")
+
+
+class CUMaskedStream:
+    """A HIP stream restricted to a share of the GPU's compute units (the
+    replacement for a per-process MPS percentage).  Usable wherever a stream is
+    accepted: ``with torch.cuda.stream(s.torch_stream): ...`` or ``stream=s``."""
+
+    def __init__(self, lo_percent: int, hi_percent: int):
+        import ctypes as _c
+        handle = _c.c_void_p()
+        ncu = _c.c_int32()
+        rc = _lib.attn().mux_stream_create_cu_range(_c.byref(handle), int(lo_percent), int(hi_percent), _c.byref(ncu))
+        _lib.check_attn(rc, "mux_stream_create_cu_range")
+        self.cuda_stream = handle.value
+        self.num_cus = ncu.value
+        self.lo_percent, self.hi_percent = int(lo_percent), int(hi_percent)
+        self.torch_stream = torch.cuda.ExternalStream(self.cuda_stream)
+
+    def synchronize(self):
+        self.torch_stream.synchronize()
+
+    def close(self):
+        if self.cuda_stream:
+            _lib.attn().mux_stream_destroy(self.cuda_stream)
+            self.cuda_stream = None
+
+
+def device_cu_info():
+    import ctypes as _c
+    out = (_c.c_int32 * 2)()
+    _lib.check_attn(_lib.attn().mux_device_cu_info(out), "mux_device_cu_info")
+    return int(out[0]), int(out[1])

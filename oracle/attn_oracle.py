@@ -177,3 +177,27 @@ def decode_bytes(context_lens, num_q_heads, num_kv_heads, block_size, head_size=
 
 def cache_write_bytes(num_tokens, num_kv_heads, head_size=HEAD_SIZE, e=2):
     return num_tokens * num_kv_heads * (2 * head_size * e + 2 * head_size * e + 8)
+
+
+# ---- rotary position embedding ---------------------------------------------------
+
+def rotary_neox(positions, q, k, rotary_dim=HEAD_SIZE, base=10000.0, head_size=HEAD_SIZE):
+    """Textbook NeoX-style RoPE (the reference constructs its attention layer
+    with rotary_dim = head_dim, base = rope_theta,
+    muxserve/flexserver/models/llama.py:138-147): for pair index i < r/2 with
+    angle p * base^(-2i/r),  (x_i, x_{i+r/2}) -> (x_i cos - x_{i+r/2} sin,
+    x_{i+r/2} cos + x_i sin).  fp64 angles, fp32 arithmetic; returns fp32
+    copies of q and k ([T, H*head_size])."""
+    T = positions.shape[0]
+    half = rotary_dim // 2
+    inv_freq = 1.0 / (base ** (torch.arange(0, rotary_dim, 2, dtype=torch.float64) / rotary_dim))
+    ang = positions.double()[:, None] * inv_freq[None, :]              # [T, half]
+    cos, sin = ang.cos().float()[:, None, :], ang.sin().float()[:, None, :]
+    outs = []
+    for t in (q, k):
+        x = t[:T].float().reshape(T, -1, head_size).clone()
+        a, b = x[..., :half].clone(), x[..., half:rotary_dim].clone()
+        x[..., :half] = a * cos - b * sin
+        x[..., half:rotary_dim] = b * cos + a * sin
+        outs.append(x.reshape(T, -1))
+    return outs[0], outs[1]

@@ -206,3 +206,31 @@ def test_workload_generators_are_seeded_and_head_granular():
     assert [m.batch for m in ms] == [32, 16, 8] and [m.num_kv_heads for m in ms] == [32, 40, 52]
     for m in ms:
         assert m.context_lens.min() >= 16 and m.context_lens.max() <= 2048
+
+
+def test_rotary_oracle_is_a_complex_rotation():
+    """NeoX RoPE pairs (x_i, x_{i+64}) and multiplies x_i + j x_{i+64} by
+    exp(j p f_i): checked with complex arithmetic, plus position 0 = identity,
+    norm preservation and the relative-position property of q.k."""
+    g = torch.Generator().manual_seed(7)
+    T, H = 6, 3
+    pos = torch.tensor([0, 1, 2, 17, 300, 2047])
+    q = torch.randn((T, H * D), generator=g).half()
+    k = torch.randn((T, 2 * D), generator=g).half()
+    rq, rk = orc.rotary_neox(pos, q, k, rotary_dim=D, base=10000.0)
+    f = 10000.0 ** (-torch.arange(0, D, 2, dtype=torch.float64) / D)
+    x = q.double().reshape(T, H, D)
+    z = torch.complex(x[..., :64], x[..., 64:]) * torch.polar(torch.ones(T, 64, dtype=torch.float64),
+                                                               pos.double()[:, None] * f)[:, None, :]
+    want = torch.cat([z.real, z.imag], dim=-1).reshape(T, H * D)
+    assert torch.allclose(rq.double(), want, atol=2e-6)
+    assert torch.equal(rq[0], q[0].float())                                  # position 0
+    assert torch.allclose(rq.reshape(T, H, D).norm(dim=-1), q.float().reshape(T, H, D).norm(dim=-1), rtol=1e-5)
+    # <rope(a, m), rope(b, n)> depends only on m - n
+    a = torch.randn((1, D), generator=g)
+    b = torch.randn((1, D), generator=g)
+    def dot(m, n):
+        ra, _ = orc.rotary_neox(torch.tensor([m]), a, a)
+        rb, _ = orc.rotary_neox(torch.tensor([n]), b, b)
+        return float((ra * rb).sum())
+    assert abs(dot(5, 2) - dot(103, 100)) < 1e-3 and abs(dot(5, 2) - dot(6, 2)) > 1e-4
