@@ -44,6 +44,10 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-hint", action="store_true", help="do not pass the host-side sum of context lengths")
     ap.add_argument("--unfused", action="store_true", help="one launch per model instead of one fused launch")
+    ap.add_argument("--workload", default="mixed3_decode",
+                    choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long"],
+                    help="mixed3_decode is the headline metric; the others are the remaining synthetic "
+                         "shapes, each printing its own JSON line")
     return ap.parse_args()
 
 
@@ -89,12 +93,229 @@ def cpu_baseline(models, k_pool, v_pool, block_size, budget_s=12.0):
     }
 
 
+def _time(fn, steps, warmup, stream=None):
+    """Average milliseconds per call of fn(i), HIP events on `stream` (torch's
+    current stream if None)."""
+    import torch
+    st = stream if stream is not None else torch.cuda.current_stream()
+    for i in range(warmup):
+        fn(i)
+    st.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(st)
+    for i in range(steps):
+        fn(i)
+    e1.record(st)
+    e1.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def _line(metric, value, unit, args, ms, config, roofline, dtype="f16", higher=True):
+    return {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": higher, "scaling": "weak",
+            "vs_baseline": None, "dtype": dtype, "data": "synthetic", "config": config, "roofline": roofline}
+
+
+def bench_prefill3(args):
+    """Config 3: causal prefill attention (MFMA) of 16 prompts per model, then
+    the cache write of the same tokens into head-wise slot mappings."""
+    import torch
+    from muxserve_amd import ops, workloads
+    from muxserve_amd.pool import HEAD_SIZE as D, allocate_gpu_cache
+    from oracle import attn_oracle as orc
+    dev, bs = "cuda:0", 16
+    models = workloads.config3(seed=args.seed)
+    total_blocks = sum(int(((m.prompt_lens + bs - 1) // bs).sum()) * m.num_kv_heads for m in models)
+    N = total_blocks + 4096
+    ids = np.random.Generator(np.random.PCG64(args.seed)).permutation(N)
+    k_pool, v_pool = allocate_gpu_cache(N, bs, dev)
+    g = torch.Generator().manual_seed(args.seed)
+    work, cur, flops, wbytes, tokens = [], 0, 0.0, 0, 0
+    for m in models:
+        T, Hq, Hkv = m.num_tokens, m.num_q_heads, m.num_kv_heads
+        pad = (T + 7) // 8 * 8
+        qkv = torch.randn((pad, (Hq + 2 * Hkv) * D), generator=g).half().to(dev)
+        q, k, v = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+        out = torch.empty((pad, Hq * D), dtype=torch.float16, device=dev)
+        cu = torch.from_numpy(m.cu_seqlens()).to(dev)
+        slots, used = workloads.prefill_slot_mapping(m.prompt_lens, Hkv, bs, ids[cur:])
+        cur += used
+        work.append((m, q, k, v, out, cu, torch.from_numpy(slots).to(dev), T))
+        flops += 4.0 * Hq * D * float((m.prompt_lens.astype(np.float64) * (m.prompt_lens + 1) / 2).sum())
+        wbytes += orc.cache_write_bytes(T, Hkv)
+        tokens += T
+
+    def attn(_):
+        for m, q, k, v, out, cu, slots, T in work:
+            ops.prefill_causal(out, q, k, v, cu, int(m.prompt_lens.max()), m.scale, m.num_kv_heads)
+
+    def write(_):
+        for m, q, k, v, out, cu, slots, T in work:
+            ops.reshape_and_cache(k, v, k_pool, v_pool, slots, num_tokens=T)
+
+    ms_a = _time(attn, args.steps, args.warmup)
+    ms_w = _time(write, args.steps, args.warmup)
+    tf = flops / (ms_a * 1e-3) / 1e12
+    gbs = wbytes / (ms_w * 1e-3) / 1e9
+    cfg = {"workload": "prefill3", "prompts_per_model": 16, "tokens": tokens, "flops": flops,
+           "cache_write_ms": ms_w, "cache_write_gbs": gbs, "cache_write_frac_of_hbm": gbs / HBM_PEAK_GBS}
+    roof = {"bound": "mfma", "achieved": tf, "peak": 2500.0, "unit": "TFLOP/s", "frac": tf / 2500.0,
+            "traffic": None, "kernel": "prefill_causal_kernel<F16>"}
+    return _line("prefill causal attention tokens/s (3 models, 16 prompts each)", tokens / (ms_a * 1e-3),
+                 "tokens/s", args, ms_a, cfg, roof)
+
+
+def bench_cache_write(args):
+    """reshape_and_cache alone: decode-shaped (one token per sequence, the three
+    models of the mix) and prefill-shaped (30B shape, 4 x 1024 tokens)."""
+    import torch
+    from muxserve_amd import ops, workloads
+    from muxserve_amd.pool import HEAD_SIZE as D, allocate_gpu_cache
+    from oracle import attn_oracle as orc
+    dev, bs = "cuda:0", 16
+    N = 1 << 20
+    k_pool, v_pool = allocate_gpu_cache(N, bs, dev)
+    rng = np.random.Generator(np.random.PCG64(args.seed))
+    g = torch.Generator().manual_seed(args.seed)
+    out = {}
+    # decode-shaped: random distinct slots
+    dec = []
+    for (hk, b) in ((32, 32), (40, 16), (52, 8)):
+        slots = rng.choice(N * bs, size=b * hk, replace=False).reshape(b, 1, hk).astype(np.int64)
+        kv = torch.randn((b, 2 * hk * D), generator=g).half().to(dev)
+        dec.append((kv[:, :hk * D], kv[:, hk * D:], torch.from_numpy(slots).to(dev), b, hk))
+    ms_d = _time(lambda _: [ops.reshape_and_cache(k, v, k_pool, v_pool, s) for k, v, s, b, hk in dec],
+                 args.steps, args.warmup)
+    bytes_d = sum(orc.cache_write_bytes(b, hk) for *_, b, hk in dec)
+    # prefill-shaped
+    lens = np.full(4, 1024)
+    slots, _ = workloads.prefill_slot_mapping(lens, 52, bs, rng.permutation(N))
+    T = int(lens.sum())
+    kv = torch.randn((T, 2 * 52 * D), generator=g).half().to(dev)
+    dslots = torch.from_numpy(slots).to(dev)
+    ms_p = _time(lambda _: ops.reshape_and_cache(kv[:, :52 * D], kv[:, 52 * D:], k_pool, v_pool, dslots),
+                 args.steps, args.warmup)
+    bytes_p = orc.cache_write_bytes(T, 52)
+    gbs = bytes_p / (ms_p * 1e-3) / 1e9
+    cfg = {"workload": "cache_write", "prefill_shape": "52 heads x 4096 tokens", "prefill_bytes": bytes_p,
+           "decode_shape": "7b/13b/30b, 56 tokens, three launches", "decode_ms": ms_d, "decode_bytes": bytes_d,
+           "decode_gbs": bytes_d / (ms_d * 1e-3) / 1e9}
+    roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+            "traffic": None, "kernel": "reshape_and_cache_kernel"}
+    return _line("KV-cache write tokens/s (prefill-shaped, 52 heads)", T / (ms_p * 1e-3), "tokens/s", args, ms_p,
+                 cfg, roof, dtype="u16")
+
+
+def bench_colocated(args):
+    """Config 4: a 30B-shaped prefill on 40% of the CUs concurrently with a
+    7B-shaped decode on the other 60%, via CU-masked streams."""
+    import torch
+    from muxserve_amd import ops, workloads
+    from muxserve_amd.pool import HEAD_SIZE as D, allocate_gpu_cache, num_gpu_blocks
+    from oracle import attn_oracle as orc
+    dev, bs = "cuda:0", 16
+    N = num_gpu_blocks(args.pool_util, torch.cuda.get_device_properties(0).total_memory, bs)
+    k_pool, v_pool = allocate_gpu_cache(N, bs, dev)
+    rng = np.random.Generator(np.random.PCG64(args.seed))
+    g = torch.Generator().manual_seed(args.seed)
+    # decode: 7B shape, batch 64, ctx U[512, 1024]; a few rotating batches
+    dsets = []
+    for i in range(4):
+        ctx = rng.integers(512, 1025, size=64).astype(np.int32)
+        need = int(((ctx + bs - 1) // bs).sum()) * 32
+        bt, _ = workloads.build_tables(ctx, 32, bs, rng.choice(N, size=need, replace=False))
+        m = workloads.DecodeModel("7b", 32, 32, ctx, bt).to_device(dev, torch.float16, seed=i)
+        dsets.append(m)
+    dbytes = float(np.mean([orc.decode_bytes(m.context_lens, 32, 32, bs) for m in dsets]))
+    # prefill: 30B shape, 4 prompts x 1024 tokens
+    T = 4096
+    qkv = torch.randn((T, 3 * 52 * D), generator=g).half().to(dev)
+    q, k, v = qkv.split([52 * D] * 3, dim=-1)
+    pout = torch.empty((T, 52 * D), dtype=torch.float16, device=dev)
+    cu = torch.tensor([0, 1024, 2048, 3072, 4096], dtype=torch.int32, device=dev)
+    pflops = 4.0 * 52 * D * 4 * (1024 * 1025 / 2)
+    s_pre, s_dec = ops.CUMaskedStream(0, 40), ops.CUMaskedStream(40, 100)
+
+    def decode(i, stream=None):
+        m = dsets[i % len(dsets)]
+        ops.paged_decode(m.out, m.q, k_pool, v_pool, m.d_block_tables, m.d_context_lens, m.max_context_len,
+                         m.scale, total_context_len=int(m.context_lens.sum()), stream=stream)
+
+    def prefill(i, stream=None):
+        ops.prefill_causal(pout, q, k, v, cu, 1024, D ** -0.5, 52, stream=stream)
+
+    steps, warm = args.steps, args.warmup
+    res = {"decode_alone_full_ms": _time(decode, steps, warm), "prefill_alone_full_ms": _time(prefill, steps, warm)}
+    res["decode_alone_60pct_ms"] = _time(lambda i: decode(i, s_dec), steps, warm, s_dec.torch_stream)
+    res["prefill_alone_40pct_ms"] = _time(lambda i: prefill(i, s_pre), steps, warm, s_pre.torch_stream)
+    # concurrent: keep both streams busy; each is timed on its own stream
+    n_pre = max(4, int(steps * res["decode_alone_60pct_ms"] / res["prefill_alone_40pct_ms"]) + 2)
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+    ev[0].record(s_dec.torch_stream)
+    ev[2].record(s_pre.torch_stream)
+    done_pre = 0
+    for i in range(steps):
+        decode(i, s_dec)
+        while done_pre < (i + 1) * n_pre // steps:
+            prefill(done_pre, s_pre)
+            done_pre += 1
+    ev[1].record(s_dec.torch_stream)
+    ev[3].record(s_pre.torch_stream)
+    torch.cuda.synchronize()
+    res["decode_concurrent_ms"] = ev[0].elapsed_time(ev[1]) / steps
+    res["prefill_concurrent_ms"] = ev[2].elapsed_time(ev[3]) / max(1, done_pre)
+    res["cus"] = [s_pre.num_cus, s_dec.num_cus]
+    gbs = dbytes / (res["decode_concurrent_ms"] * 1e-3) / 1e9
+    res.update({"workload": "colocated", "decode_bytes": dbytes, "prefill_flops": pflops,
+                "prefill_concurrent_tflops": pflops / (res["prefill_concurrent_ms"] * 1e-3) / 1e12,
+                "decode_alone_full_gbs": dbytes / (res["decode_alone_full_ms"] * 1e-3) / 1e9})
+    roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+            "traffic": None, "kernel": "paged_decode_kernel<F16,16,1,4> on 60% of CUs, prefill on the rest"}
+    return _line("decode attn tokens/s on 60% of CUs while a prefill runs on 40%", 64 / (res["decode_concurrent_ms"] * 1e-3),
+                 "tokens/s", args, res["decode_concurrent_ms"], res, roof)
+
+
+def bench_gqa_long(args):
+    """Config 5: 64 query heads over 8 kv heads, bf16, batch 64, ctx U[2048, 8192]."""
+    import torch
+    from muxserve_amd import ops, workloads
+    from muxserve_amd.pool import allocate_gpu_cache
+    from oracle import attn_oracle as orc
+    dev, bs = "cuda:0", 16
+    N = int(200e9) // 8192 // 128 * 128
+    k_pool, v_pool = allocate_gpu_cache(N, bs, dev, dtype=torch.bfloat16)
+    sets = []
+    for i in range(3):
+        m = workloads.config5(seed=args.seed + i, num_pool_blocks=N)[0][0].to_device(dev, torch.bfloat16, seed=i)
+        sets.append(m)
+
+    def step(i):
+        m = sets[i % len(sets)]
+        ops.paged_decode(m.out, m.q, k_pool, v_pool, m.d_block_tables, m.d_context_lens, m.max_context_len,
+                         m.scale, partition_size=args.partition, total_context_len=int(m.context_lens.sum()))
+
+    ms = _time(step, args.steps, args.warmup)
+    nbytes = float(np.mean([orc.decode_bytes(m.context_lens, 64, 8, bs) for m in sets]))
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    cfg = {"workload": "gqa_long", "shape": "Hq64/Hkv8, B=64, ctx U[2048,8192], bf16", "pool_gb": round(N * 8192 / 1e9, 1),
+           "bytes_per_step": int(nbytes), "partition": args.partition}
+    roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+            "traffic": None, "kernel": "paged_decode_kernel<BF16,16,8,4>"}
+    return _line("long-context GQA decode attn tokens/s", 64 / (ms * 1e-3), "tokens/s", args, ms, cfg, roof, dtype="bf16")
+
+
 def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives or sharding); use --gpus 1",
               file=sys.stderr)
         sys.exit(2)
+    other = {"prefill3": bench_prefill3, "cache_write": bench_cache_write, "colocated": bench_colocated,
+             "gqa_long": bench_gqa_long}
+    if args.workload in other:
+        print(json.dumps(other[args.workload](args)))
+        return
 
     import torch
     from muxserve_amd import ops, workloads

@@ -41,6 +41,13 @@ __device__ __forceinline__ half2_t as_half2(uint32_t u) {
   return c.h;
 }
 
+typedef __bf16 bf162_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ bf162_t as_bf162(uint32_t u) {
+  union { uint32_t u; bf162_t h; } c;
+  c.u = u;
+  return c.h;
+}
+
 // fp32 -> bf16 bits, round to nearest even (NaN kept quiet).
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
   uint32_t u = __float_as_uint(f);
@@ -67,8 +74,7 @@ __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
   if constexpr (__is_same(T, F16)) {
     return __builtin_amdgcn_fdot2(as_half2(a), as_half2(b), acc, false);
   } else {
-    acc = __builtin_fmaf(bf16_lo(a), bf16_lo(b), acc);
-    return __builtin_fmaf(bf16_hi(a), bf16_hi(b), acc);
+    return __builtin_amdgcn_fdot2_f32_bf16(as_bf162(a), as_bf162(b), acc, false);   // v_dot2c_f32_bf16
   }
 }
 
