@@ -30,6 +30,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes moved per algorithmic byte by the decode kernel on this workload,
+# from the FETCH_SIZE / WRITE_SIZE counter passes summarised in
+# profiles/paged_decode_mixed3_hbm_traffic.txt (421.0 MB measured / 410.6 MB).
+MIXED3_TRAFFIC_RATIO = 1.025
 
 
 def parse():
@@ -402,8 +406,9 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
-            "kernel": "paged_decode_kernel<F16,16,1>",
+            "traffic": avg_bytes * MIXED3_TRAFFIC_RATIO if not args.unfused else None,
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiles/paged_decode_mixed3_hbm_traffic.txt",
+            "kernel": "paged_decode_kernel<F16,16,1,4>",
             "event_ms_per_step": ev_ms,
         },
     }
