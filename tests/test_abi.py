@@ -1,0 +1,62 @@
+"""The two C-ABI libraries load without a GPU and export every entry point the
+headers under include/ declare (no compute calls here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from muxserve_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DECL = re.compile(r"^\s*(?:[A-Za-z_][\w\s\*]*?)\b(mux_\w+)\s*\(", re.M)
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)          # drop comments
+    return sorted(set(DECL.findall(text)))
+
+
+@pytest.mark.parametrize("header,loader,path", [
+    ("muxserve_host.h", _lib.host, _lib.HOST_LIB_PATH),
+    ("muxserve_attn.h", _lib.attn, _lib.ATTN_LIB_PATH),
+])
+def test_library_exports_every_declared_symbol(header, loader, path):
+    names = _declared(header)
+    assert len(names) >= 10, names
+    lib = loader()
+    raw = ctypes.CDLL(path)
+    for n in names:
+        assert hasattr(raw, n), f"{n} declared in include/{header} but not exported by {os.path.basename(path)}"
+    # every declared symbol also has a typed binding
+    typed = set(_lib.ATTN_SIGNATURES) if header == "muxserve_attn.h" else None
+    if typed is not None:
+        assert set(names) <= typed, sorted(set(names) - typed)
+    assert lib is loader()      # cached handle
+
+
+def test_version_and_error_entry_points_work_without_a_gpu():
+    lib = _lib.attn()
+    assert lib.mux_attn_version() >= 100
+    assert lib.mux_last_hip_error() == 0
+
+
+def test_missing_library_fails_loudly(tmp_path, monkeypatch):
+    monkeypatch.setattr(_lib, "_attn", None)
+    monkeypatch.setattr(_lib, "ATTN_LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.MuxLibraryMissing):
+        _lib.attn()
+
+
+def test_decode_rejects_malformed_arguments_on_the_host_side():
+    """Validation happens before any launch, so it can be exercised without a GPU."""
+    lib = _lib.attn()
+    item = _lib.MuxDecodeItem()
+    rc = lib.mux_multi_decode(ctypes.addressof(item), 1, 16, 16, 8, 128, 16, 0, 0, None, 0, None)
+    assert rc == -1          # null q/out/tables
+    rc = lib.mux_multi_decode(ctypes.addressof(item), 9, 16, 16, 8, 128, 16, 0, 0, None, 0, None)
+    assert rc == -1          # too many items
+    rc = lib.mux_reshape_and_cache(16, 16, 128, 16, 16, 8, 16, 0, 1, 4, 1, 64, 16, 0, None)
+    assert rc == -2          # head size other than 128
+    assert lib.mux_stream_create_cu_range(None, 0, 50, None) == -1
