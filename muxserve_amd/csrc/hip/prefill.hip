@@ -30,7 +30,7 @@ typedef float v16f32 __attribute__((ext_vector_type(16)));
 constexpr int kBM = 128;                 // query rows per workgroup
 constexpr int kBN = 64;                  // keys per tile
 constexpr int kKRow = kHeadSize + 8;     // K tile row length in elements (272 B: 16-byte frags, rows 4 banks apart)
-constexpr int kVRow = kBN + 8;           // V^T tile row length in elements (144 B)
+constexpr int kVRow = kBN + 4;           // V^T tile row length in elements (136 B: 8-byte frags, rows 2 banks apart)
 
 union Frag {
   uint4 u;
@@ -61,7 +61,7 @@ struct PrefillParams {
 };
 
 template <typename T>
-__global__ __launch_bounds__(256) void prefill_causal_kernel(const PrefillParams P) {
+__global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillParams P) {
   constexpr int D = kHeadSize;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[kBN * kKRow];
   __shared__ __attribute__((aligned(16))) uint16_t Vt[D * kVRow];
@@ -172,26 +172,26 @@ __global__ __launch_bounds__(256) void prefill_causal_kernel(const PrefillParams
     }
 
     // ---- softmax over keys, per query column --------------------------------------
-    // register i of block kb is key k0 + 32 kb + 8 (i/4) + 4 half + i%4
+    // register i of block kb is key k0 + 32 kb + 8 (i/4) + 4 half + i%4.
+    // Raw scores stay unscaled; scale (> 0) is folded into the exponent:
+    // p = exp2(s * scale_log2 - m * scale_log2).
     float mx = -INFINITY;
     const bool diag = k0 + kBN - 1 > wq0;   // some (key, q) pair of this wave's tile is masked
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        float sv = sacc[kb][i] * P.scale_log2;
         if (diag) {
           const int key = k0 + 32 * kb + 8 * (i / 4) + 4 * half + (i % 4);
-          if (key > my_q) sv = -INFINITY;
+          if (key > my_q) sacc[kb][i] = -INFINITY;
         }
-        sacc[kb][i] = sv;
-        mx = fmaxf(mx, sv);
+        mx = fmaxf(mx, sacc[kb][i]);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const float m_new = fmaxf(m_run, mx);
     // Rows past the prompt may have no valid key at all; keep them finite.
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = fast_exp2(m_run - m_use);
+    const float neg_m = -m_use * P.scale_log2;
     float psum = 0.f;
     Frag pf[4];                          // B fragments: [kb][step] -> index 2 kb + st
     // bf16 keeps only 8 mantissa bits of a probability, which alone would cost
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(256) void prefill_causal_kernel(const PrefillParams
       float p[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        p[i] = fast_exp2(sacc[kb][i] - m_use);
+        p[i] = fast_exp2(__builtin_fmaf(sacc[kb][i], P.scale_log2, neg_m));
         psum += p[i];
       }
 #pragma unroll
@@ -220,12 +220,18 @@ __global__ __launch_bounds__(256) void prefill_causal_kernel(const PrefillParams
         }
       }
     }
-    l_run = l_run * alpha + psum;
+    // The running max rises only in the first tiles of a row; skip the rescale
+    // of the 64 accumulators when no lane of the wave needs it.
+    if (__builtin_amdgcn_ballot_w64(m_use > m_run) != 0) {
+      const float alpha = fast_exp2((m_run - m_use) * P.scale_log2);
+      l_run *= alpha;
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[mb][i] *= alpha;
+    }
+    l_run += psum;
     m_run = m_use;
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[mb][i] *= alpha;
 
     // ---- O^T += V^T . P^T ---------------------------------------------------------------
     // k-slot j of lane half h in step (kb, st) is key 32 kb + 16 st + 8 (j/4) + 4 h + j%4
