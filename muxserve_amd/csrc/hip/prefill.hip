@@ -26,6 +26,8 @@ namespace mux {
 typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
 typedef __bf16 v8bf16 __attribute__((ext_vector_type(8)));
 typedef float v16f32 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kBM = 128;                 // query rows per workgroup
 constexpr int kBN = 64;                  // keys per tile
@@ -33,7 +35,7 @@ constexpr int kKRow = kHeadSize + 8;     // K tile row length in elements (272 B
 constexpr int kVRow = kBN + 4;           // V^T tile row length in elements (136 B: 8-byte frags, rows 2 banks apart)
 
 union Frag {
-  uint4 u;
+  u32x4 u;
   v8f16 h;
   v8bf16 b;
 };
@@ -44,10 +46,21 @@ __device__ __forceinline__ v16f32 mfma(const Frag &a, const Frag &b, v16f32 c) {
   else return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.b, b.b, c, 0, 0, 0);
 }
 
-// Two fp32 -> one packed pair in storage type T.
+// Two fp32 -> one packed pair in storage type T, round to nearest even
+// (one v_cvt_pk_f16_f32 / v_cvt_pk_bf16_f32).
+typedef float float2_t __attribute__((ext_vector_type(2)));
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-  return static_cast<uint32_t>(to_storage<T>(lo)) | (static_cast<uint32_t>(to_storage<T>(hi)) << 16);
+  const float2_t x = {lo, hi};
+  if constexpr (__is_same(T, F16)) {
+    union { half2_t h; uint32_t u; } c;
+    c.h = __builtin_convertvector(x, half2_t);
+    return c.u;
+  } else {
+    union { bf162_t h; uint32_t u; } c;
+    c.h = __builtin_convertvector(x, bf162_t);
+    return c.u;
+  }
 }
 
 struct PrefillParams {
@@ -56,7 +69,9 @@ struct PrefillParams {
   int64_t out_stride, q_stride, kv_stride;
   const int32_t *cu_seqlens;
   int32_t ratio;          // query heads per kv head
-  int32_t q_tiles;        // grid.x
+  int32_t q_tiles;        // 128-row query tiles per prompt (of the longest prompt)
+  int32_t num_kv_heads;
+  int32_t num_groups;     // (prompt, kv head) pairs
   float scale_log2;
 };
 
@@ -69,13 +84,22 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int hq = blockIdx.y;
-  const int hk = hq / P.ratio;
-  const int prompt = blockIdx.z;
+  // Workgroups are dealt to the 8 XCDs round-robin by id, and each XCD has its
+  // own L2.  All workgroups that read the same K/V - the query tiles and query
+  // heads of one (prompt, kv head) group - are therefore given ids that are
+  // equal mod 8, and groups go round-robin over the XCDs.
+  const int per_group = P.ratio * P.q_tiles;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int group = (slot / per_group) * 8 + xcd;
+  if (group >= P.num_groups) return;
+  const int in_group = slot % per_group;
+  const int prompt = group / P.num_kv_heads;
+  const int hk = group % P.num_kv_heads;
+  const int hq = hk * P.ratio + in_group / P.q_tiles;
   const int seq_begin = P.cu_seqlens[prompt];
   const int len = P.cu_seqlens[prompt + 1] - seq_begin;
   // Heaviest tiles (most keys) first.
-  const int q0 = (P.q_tiles - 1 - static_cast<int>(blockIdx.x)) * kBM;
+  const int q0 = (P.q_tiles - 1 - in_group % P.q_tiles) * kBM;
   if (q0 >= len) return;
 
   const int qcol = lane & 31;            // this lane's query column / fragment row
@@ -89,7 +113,7 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
     const bool ok = my_q < len;
     const uint16_t *qp = P.q + static_cast<int64_t>(seq_begin + (ok ? my_q : 0)) * P.q_stride + hq * D + 8 * half;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) qf[s].u = ok ? *reinterpret_cast<const uint4 *>(qp + 16 * s) : make_uint4(0, 0, 0, 0);
+    for (int s = 0; s < 8; ++s) qf[s].u = ok ? *reinterpret_cast<const u32x4 *>(qp + 16 * s) : u32x4{0, 0, 0, 0};
   }
 
   v16f32 oacc[4];                        // O^T[d = 32 mb + ...][q]
@@ -105,32 +129,41 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
 
   // Global -> register staging of one K/V tile.  K: thread takes chunk
   // (key = tid/16 + 16 i, dchunk = tid%16).  V: thread takes keys 4 kg .. 4 kg+3
-  // (kg = tid%16) of dchunk vc = tid/16.
+  // (kg = tid%16) of dchunk vc = tid/16.  Addresses are a uniform base plus a
+  // 32-bit per-thread byte offset that advances by one tile per load.  Rows past
+  // the prompt re-read its last row: finite data whose probability is exactly 0
+  // (such a key is in the future of every valid query).
   const int kc = tid & 15, kk = tid >> 4;
   const int vg = tid & 15, vc = tid >> 4;
-  uint4 kst[4], vst[4];
-  auto load_tile = [&](int t) {
-    const int k0 = t * kBN;
+  const uint32_t row_bytes = static_cast<uint32_t>(P.kv_stride) * 2u;
+  const char *kbase = reinterpret_cast<const char *>(P.k + static_cast<int64_t>(seq_begin) * P.kv_stride + hk * D);
+  const char *vbase = reinterpret_cast<const char *>(P.v + static_cast<int64_t>(seq_begin) * P.kv_stride + hk * D);
+  uint32_t koff[4], voff[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    koff[i] = static_cast<uint32_t>(kk + 16 * i) * row_bytes + 16u * kc;
+    voff[i] = static_cast<uint32_t>(4 * vg + i) * row_bytes + 16u * vc;
+  }
+  const uint32_t tile_bytes = kBN * row_bytes;
+  const uint32_t last_row = static_cast<uint32_t>(len - 1) * row_bytes;
+  const uint32_t kmax = last_row + 16u * kc, vmax = last_row + 16u * vc;
+  u32x4 kst[4], vst[4];
+  auto load_tile = [&]() {                 // loads the next tile in sequence
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int key = k0 + kk + 16 * i;
-      kst[i] = key < len ? *reinterpret_cast<const uint4 *>(
-                               P.k + static_cast<int64_t>(seq_begin + key) * P.kv_stride + hk * D + 8 * kc)
-                         : make_uint4(0, 0, 0, 0);
+      kst[i] = *reinterpret_cast<const u32x4 *>(kbase + min(koff[i], kmax));
+      koff[i] += tile_bytes;
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int key = k0 + 4 * vg + i;
-      // Rows past the prompt are zero so that 0 * garbage cannot make a NaN.
-      vst[i] = key < len ? *reinterpret_cast<const uint4 *>(
-                               P.v + static_cast<int64_t>(seq_begin + key) * P.kv_stride + hk * D + 8 * vc)
-                         : make_uint4(0, 0, 0, 0);
+      vst[i] = *reinterpret_cast<const u32x4 *>(vbase + min(voff[i], vmax));
+      voff[i] += tile_bytes;
     }
   };
   auto store_tile = [&]() {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      *reinterpret_cast<uint4 *>(&Ks[(kk + 16 * i) * kKRow + 8 * kc]) = kst[i];
+      *reinterpret_cast<u32x4 *>(&Ks[(kk + 16 * i) * kKRow + 8 * kc]) = kst[i];
     // 4 keys x 8 dims -> 8 rows of V^T, 4 keys (8 bytes) each.
     const uint32_t a[4][4] = {{vst[0].x, vst[0].y, vst[0].z, vst[0].w},
                               {vst[1].x, vst[1].y, vst[1].z, vst[1].w},
@@ -143,31 +176,43 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
       const uint32_t lo23 = __builtin_amdgcn_perm(a[3][w], a[2][w], 0x05040100u);
       const uint32_t hi01 = __builtin_amdgcn_perm(a[1][w], a[0][w], 0x07060302u);
       const uint32_t hi23 = __builtin_amdgcn_perm(a[3][w], a[2][w], 0x07060302u);
-      *reinterpret_cast<uint2 *>(&Vt[(8 * vc + 2 * w) * kVRow + 4 * vg]) = make_uint2(lo01, lo23);
-      *reinterpret_cast<uint2 *>(&Vt[(8 * vc + 2 * w + 1) * kVRow + 4 * vg]) = make_uint2(hi01, hi23);
+      *reinterpret_cast<u32x2 *>(&Vt[(8 * vc + 2 * w) * kVRow + 4 * vg]) = u32x2{lo01, lo23};
+      *reinterpret_cast<u32x2 *>(&Vt[(8 * vc + 2 * w + 1) * kVRow + 4 * vg]) = u32x2{hi01, hi23};
     }
   };
 
-  load_tile(0);
+  load_tile();
   for (int t = 0; t < n_tiles; ++t) {
     const int k0 = t * kBN;
     __syncthreads();                     // everyone is done reading the previous tile
     store_tile();
     __syncthreads();
-    if (t + 1 < n_tiles) load_tile(t + 1);
+    if (t + 1 < n_tiles) load_tile();
     if (k0 > wq0 + 31) continue;         // every key of the tile is in this wave's future
 
     // ---- S^T = K . Q^T : two 32-key blocks ------------------------------------------
+    // LDS fragment reads run kDepth steps ahead of the MFMAs that consume them.
+    constexpr int kDepth = 4;
     v16f32 sacc[2];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
+    {
+      const uint16_t *kr = &Ks[qcol * kKRow + 8 * half];
+      Frag ring[kDepth];
 #pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        Frag kf;
-        kf.u = *reinterpret_cast<const uint4 *>(&Ks[(32 * kb + qcol) * kKRow + 16 * s + 8 * half]);
-        sacc[kb] = mfma<T>(kf, qf[s], sacc[kb]);
+      for (int j = 0; j < kDepth; ++j)
+        ring[j].u = *reinterpret_cast<const u32x4 *>(kr + (j / 8) * 32 * kKRow + 16 * (j % 8));
+      __builtin_amdgcn_sched_barrier(0);   // keep the scheduler from sinking the reads to their uses
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        sacc[j / 8] = mfma<T>(ring[j % kDepth], qf[j % 8], sacc[j / 8]);
+        if (j + kDepth < 16) {
+          const int n = j + kDepth;
+          ring[j % kDepth].u = *reinterpret_cast<const u32x4 *>(kr + (n / 8) * 32 * kKRow + 16 * (n % 8));
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
 
@@ -175,18 +220,20 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
     // register i of block kb is key k0 + 32 kb + 8 (i/4) + 4 half + i%4.
     // Raw scores stay unscaled; scale (> 0) is folded into the exponent:
     // p = exp2(s * scale_log2 - m * scale_log2).
+    // Exactly one tile per wave straddles the diagonal; only it pays for the mask.
+    if (k0 + kBN - 1 > wq0) {
+      const int rel = my_q - k0 - 4 * half;   // key offset inside the tile, less this lane's share
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (32 * kb + 8 * (i / 4) + (i % 4) > rel) sacc[kb][i] = -INFINITY;
+    }
     float mx = -INFINITY;
-    const bool diag = k0 + kBN - 1 > wq0;   // some (key, q) pair of this wave's tile is masked
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        if (diag) {
-          const int key = k0 + 32 * kb + 8 * (i / 4) + 4 * half + (i % 4);
-          if (key > my_q) sacc[kb][i] = -INFINITY;
-        }
-        mx = fmaxf(mx, sacc[kb][i]);
-      }
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kb][i]);
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const float m_new = fmaxf(m_run, mx);
     // Rows past the prompt may have no valid key at all; keep them finite.
@@ -208,15 +255,15 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
       }
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
-        pf[2 * kb + st].u = make_uint4(pack2<T>(p[8 * st + 0], p[8 * st + 1]), pack2<T>(p[8 * st + 2], p[8 * st + 3]),
-                                       pack2<T>(p[8 * st + 4], p[8 * st + 5]), pack2<T>(p[8 * st + 6], p[8 * st + 7]));
+        pf[2 * kb + st].u = u32x4{pack2<T>(p[8 * st + 0], p[8 * st + 1]), pack2<T>(p[8 * st + 2], p[8 * st + 3]),
+                                       pack2<T>(p[8 * st + 4], p[8 * st + 5]), pack2<T>(p[8 * st + 6], p[8 * st + 7])};
         if constexpr (kSplitP) {
           float r[8];
 #pragma unroll
           for (int j = 0; j < 8; ++j)
             r[j] = p[8 * st + j] - __uint_as_float(static_cast<uint32_t>(f32_to_bf16_bits(p[8 * st + j])) << 16);
-          pf_lo[2 * kb + st].u = make_uint4(pack2<T>(r[0], r[1]), pack2<T>(r[2], r[3]),
-                                            pack2<T>(r[4], r[5]), pack2<T>(r[6], r[7]));
+          pf_lo[2 * kb + st].u = u32x4{pack2<T>(r[0], r[1]), pack2<T>(r[2], r[3]),
+                                            pack2<T>(r[4], r[5]), pack2<T>(r[6], r[7])};
         }
       }
     }
@@ -235,17 +282,26 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
 
     // ---- O^T += V^T . P^T ---------------------------------------------------------------
     // k-slot j of lane half h in step (kb, st) is key 32 kb + 16 st + 8 (j/4) + 4 h + j%4
+    {
+      const uint16_t *vr = &Vt[qcol * kVRow + 4 * half];
+      auto read_v = [&](int n) {         // fragment n = 4 mb + ks
+        const uint16_t *r = vr + (n / 4) * 32 * kVRow + 16 * (n % 4);
+        const u32x2 lo = *reinterpret_cast<const u32x2 *>(r);
+        const u32x2 hi = *reinterpret_cast<const u32x2 *>(r + 8);
+        Frag f;
+        f.u = u32x4{lo.x, lo.y, hi.x, hi.y};
+        return f;
+      };
+      Frag ring[kDepth];
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
+      for (int j = 0; j < kDepth; ++j) ring[j] = read_v(j);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const uint16_t *vr = &Vt[(32 * mb + qcol) * kVRow + 16 * ks + 4 * half];
-        const uint2 lo = *reinterpret_cast<const uint2 *>(vr);
-        const uint2 hi = *reinterpret_cast<const uint2 *>(vr + 8);
-        Frag vf;
-        vf.u = make_uint4(lo.x, lo.y, hi.x, hi.y);
-        oacc[mb] = mfma<T>(vf, pf[ks], oacc[mb]);
-        if constexpr (kSplitP) oacc[mb] = mfma<T>(vf, pf_lo[ks], oacc[mb]);
+      for (int j = 0; j < 16; ++j) {
+        oacc[j / 4] = mfma<T>(ring[j % kDepth], pf[j % 4], oacc[j / 4]);
+        if constexpr (kSplitP) oacc[j / 4] = mfma<T>(ring[j % kDepth], pf_lo[j % 4], oacc[j / 4]);
+        if (j + kDepth < 16) ring[j % kDepth] = read_v(j + kDepth);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   }
@@ -287,7 +343,8 @@ extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const v
   if (q_row_stride % 8 || kv_row_stride % 8 || out_row_stride % 4) return MUXA_EINVAL;
   const uintptr_t a16 = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v);
   if ((a16 & 15u) || (reinterpret_cast<uintptr_t>(out) & 7u)) return MUXA_EINVAL;
-  if (num_q_heads > 65535 || num_prompts > 65535) return MUXA_EUNSUPPORTED;
+  // K/V rows of one prompt are addressed with 32-bit byte offsets.
+  if (static_cast<int64_t>(max_prompt_len + kBM + 2 * kBN) * kv_row_stride * 2 >= (int64_t{1} << 32)) return MUXA_EUNSUPPORTED;
   if (num_prompts == 0 || max_prompt_len == 0) return MUXA_OK;
 
   PrefillParams P;
@@ -301,8 +358,12 @@ extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const v
   P.cu_seqlens = cu_seqlens;
   P.ratio = num_q_heads / num_kv_heads;
   P.q_tiles = (max_prompt_len + kBM - 1) / kBM;
+  P.num_kv_heads = num_kv_heads;
+  P.num_groups = num_prompts * num_kv_heads;
   P.scale_log2 = scale * 1.4426950408889634f;
-  const dim3 grid(P.q_tiles, num_q_heads, num_prompts);
+  const int64_t n_wg = static_cast<int64_t>((P.num_groups + 7) / 8) * 8 * P.ratio * P.q_tiles;
+  if (n_wg > 0x7fffffff) return MUXA_EUNSUPPORTED;
+  const dim3 grid(static_cast<uint32_t>(n_wg));
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == MUXA_DTYPE_F16) hipLaunchKernelGGL(prefill_causal_kernel<F16>, grid, dim3(256), 0, st, P);
   else hipLaunchKernelGGL(prefill_causal_kernel<BF16>, grid, dim3(256), 0, st, P);
