@@ -305,7 +305,7 @@ def bench_gqa_long(args):
     cfg = {"workload": "gqa_long", "shape": "Hq64/Hkv8, B=64, ctx U[2048,8192], bf16", "pool_gb": round(N * 8192 / 1e9, 1),
            "bytes_per_step": int(nbytes), "partition": args.partition}
     roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-            "traffic": None, "kernel": "paged_decode_kernel<BF16,16,8,4>"}
+            "traffic": None, "kernel": "paged_decode_gqa_kernel<BF16,16,8,4>"}
     return _line("long-context GQA decode attn tokens/s", 64 / (ms * 1e-3), "tokens/s", args, ms, cfg, roof, dtype="bf16")
 
 

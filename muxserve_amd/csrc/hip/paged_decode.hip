@@ -241,6 +241,54 @@ __device__ __forceinline__ void stash_wave_partial(float (&m)[G], float (&l)[G],
   }
 }
 
+// Combine of one head's partitions by one wave: out = sum_i w_i acc_i / sum_i w_i l_i,
+// w_i = 2^(m_i - max m).  Lane i of a 64-partition chunk holds (m_i, l_i); the
+// partial accumulators are fetched eight partitions at a time, all loads in
+// flight together (partition indices past the end re-read the last partition
+// with weight 0).
+template <typename T>
+__device__ __forceinline__ void combine_head(const DecodeItemDev &I, int seq, int hq, int n_splits, int lane) {
+  constexpr int D = kHeadSize;
+  const int64_t base = (static_cast<int64_t>(seq) * I.Hq + hq) * I.max_splits;
+  const float *ml = I.ws_ml + base * 2;
+  const float *pa = I.ws_acc + base * D;
+  float M = -INFINITY;
+  for (int c0 = 0; c0 < n_splits; c0 += 64) {
+    const int i = c0 + lane;
+    if (i < n_splits) M = fmaxf(M, coherent_load(&ml[i * 2]));
+  }
+  M = wave_max(M);
+  float Lsum = 0.f, a0 = 0.f, a1 = 0.f;
+  for (int c0 = 0; c0 < n_splits; c0 += 64) {
+    const int i = c0 + lane;
+    float wl = 0.f;
+    if (i < n_splits) {
+      wl = fast_exp2(coherent_load(&ml[i * 2]) - M);
+      Lsum += coherent_load(&ml[i * 2 + 1]) * wl;
+    }
+    const int cnt = min(64, n_splits - c0);
+    for (int k0 = 0; k0 < cnt; k0 += 8) {
+      float v0[8], v1[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int idx = min(c0 + k0 + j, n_splits - 1);
+        v0[j] = coherent_load(&pa[idx * D + lane]);
+        v1[j] = coherent_load(&pa[idx * D + 64 + lane]);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float wj = k0 + j < 64 ? lane_bcast(wl, (k0 + j) & 63) : 0.f;
+        a0 = __builtin_fmaf(v0[j], wj, a0);
+        a1 = __builtin_fmaf(v1[j], wj, a1);
+      }
+    }
+  }
+  Lsum = wave_sum(Lsum);
+  uint16_t *o = static_cast<uint16_t *>(I.out) + static_cast<int64_t>(seq) * I.out_stride + hq * D;
+  o[lane] = to_storage<T>(a0 / Lsum);
+  o[64 + lane] = to_storage<T>(a1 / Lsum);
+}
+
 // Wave 0: merge the workgroup's NW partials (lane owns dims lane and lane+64),
 // then either write the output (context fits one partition) or publish the
 // partition's partial and, if this was the last partition to arrive, combine
@@ -295,26 +343,67 @@ __device__ __forceinline__ void merge_and_write(const DecodeItemDev &I, const Un
   if (arrived != n_splits - 1) return;
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 #pragma unroll 1
-  for (int g = 0; g < G; ++g) {
-    const int hq = hq0 + g;
-    const int64_t base = (static_cast<int64_t>(u.seq) * I.Hq + hq) * I.max_splits;
-    const float *ml = I.ws_ml + base * 2;
-    const float *pa = I.ws_acc + base * D;
-    float M = -INFINITY;
-    for (int i = 0; i < n_splits; ++i) M = fmaxf(M, coherent_load(&ml[i * 2]));
-    float Lsum = 0.f, a0 = 0.f, a1 = 0.f;
-    for (int i = 0; i < n_splits; ++i) {
-      const float wgt = fast_exp2(coherent_load(&ml[i * 2]) - M);
-      Lsum += coherent_load(&ml[i * 2 + 1]) * wgt;
-      a0 += coherent_load(&pa[i * D + lane]) * wgt;
-      a1 += coherent_load(&pa[i * D + 64 + lane]) * wgt;
-    }
-    uint16_t *o = static_cast<uint16_t *>(I.out) + static_cast<int64_t>(u.seq) * I.out_stride + hq * D;
-    o[lane] = to_storage<T>(a0 / Lsum);
-    o[64 + lane] = to_storage<T>(a1 / Lsum);
-  }
+  for (int g = 0; g < G; ++g) combine_head<T>(I, u.seq, hq0 + g, n_splits, lane);
   // Ready for the next launch.
   if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The same merge, publish and combine for a group of G heads, spread over the
+// workgroup's NW waves (wave w takes heads w, w+NW, ...).  Every wave of the
+// workgroup must call it.
+template <typename T, int G, int NW>
+__device__ __forceinline__ void merge_and_write_group(const DecodeItemDev &I, const Unit &u, int partition,
+                                                      const float (*xa)[G][kHeadSize], const float (*xm)[G][2],
+                                                      int *arrival_lds, int lane, int wave) {
+  constexpr int D = kHeadSize;
+  const bool single = u.ctx <= partition;
+  const int hq0 = u.wh * G;
+#pragma unroll 1
+  for (int g = wave; g < G; g += NW) {
+    float M = xm[0][g][0];
+#pragma unroll
+    for (int k = 1; k < NW; ++k) M = fmaxf(M, xm[k][g][0]);
+    float L = 0.f, a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int k = 0; k < NW; ++k) {
+      const float wgt = fast_exp2(xm[k][g][0] - M);
+      L += xm[k][g][1] * wgt;
+      a0 += xa[k][g][lane] * wgt;
+      a1 += xa[k][g][64 + lane] * wgt;
+    }
+    const int hq = hq0 + g;
+    if (single) {
+      uint16_t *o = static_cast<uint16_t *>(I.out) + static_cast<int64_t>(u.seq) * I.out_stride + hq * D;
+      o[lane] = to_storage<T>(a0 / L);
+      o[64 + lane] = to_storage<T>(a1 / L);
+    } else {
+      const int64_t prow = (static_cast<int64_t>(u.seq) * I.Hq + hq) * I.max_splits + u.split;
+      coherent_store(&I.ws_acc[prow * D + lane], a0);
+      coherent_store(&I.ws_acc[prow * D + 64 + lane], a1);
+      if (lane == 0) {
+        coherent_store(&I.ws_ml[prow * 2], M);
+        coherent_store(&I.ws_ml[prow * 2 + 1], L);
+      }
+    }
+  }
+  if (single) return;
+
+  // Each wave waits for its own partial stores (they bypass the per-XCD L2, so
+  // completion is all that is needed), the workgroup meets, one lane announces
+  // the arrival and tells the others whether this workgroup came last.
+  const int n_splits = (u.ctx + partition - 1) / partition;
+  int32_t *counter = I.counters + static_cast<int64_t>(u.seq) * (I.Hq / G) + u.wh;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (wave == 0 && lane == 0)
+    *arrival_lds = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  if (*arrival_lds != n_splits - 1) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll 1
+  for (int g = wave; g < G; g += NW) combine_head<T>(I, u.seq, hq0 + g, n_splits, lane);
+  // Ready for the next launch.
+  if (wave == 0 && lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------
@@ -468,6 +557,283 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_kernel(const DecodeParam
   merge_and_write<T, G, NW>(I, u, partition, x_acc, x_ml, lane);
 }
 
+// ---------------------------------------------------------------------------
+// Grouped-query kernel (G >= 4 query heads per kv head): the G heads of a group
+// read the same K/V, so scores and P.V are small matrix products and go to the
+// matrix cores (v_mfma_f32_16x16x32_{f16,bf16}), with the group padded to the 16
+// columns of the instruction.  Both products are kept transposed so that a lane
+// owns ONE head (lane % 16) throughout and the softmax state is a per-lane scalar:
+//     S^T[tok][head] = K . Q^T     A = K   : lane (tok = l%16, g = l/16) holds dims
+//                                            32 s + 8 g .. +7 of its token - exactly
+//                                            the pool's 16-byte chunk (d/8, tok)
+//                                  B = Q^T : lane (head = l%16, g), same dims
+//     O^T[d][head]  += V^T . P^T   A = V^T : lane (d = 16 nb + l%16, g) holds tokens
+//                                            32 ts + 8 g .. +7 of its dim - exactly
+//                                            the pool's 16-byte chunk (d, tok/8)
+//                                  B = P^T : lane (head = l%16, g), same tokens
+// so every K and V load lands in its operand register straight from the pool.
+// The score accumulators give a lane tokens 16 tg + 4 g + i of its head; the
+// regrouping into runs of 8 tokens goes through 1 KiB of LDS per wave.
+// A wave advances 32 tokens per step with two register sets, so the loads of
+// the next step are in flight while the current one is consumed.
+// Work units, partitions, the cross-wave merge and the split combine are those
+// of the kernel above.
+// ---------------------------------------------------------------------------
+typedef _Float16 v8f16_t __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf16_t __attribute__((ext_vector_type(8)));
+typedef float v4f32_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+union Frag8 {
+  u32x4_t u;
+  v8f16_t h;
+  v8bf16_t b;
+};
+
+template <typename T>
+__device__ __forceinline__ v4f32_t mfma16(const Frag8 &a, const Frag8 &b, v4f32_t c) {
+  if constexpr (__is_same(T, F16)) return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, c, 0, 0, 0);
+  else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, c, 0, 0, 0);
+}
+
+typedef float float2v_t __attribute__((ext_vector_type(2)));
+template <typename T>
+__device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
+  const float2v_t x = {lo, hi};
+  if constexpr (__is_same(T, F16)) {
+    union { half2_t h; uint32_t u; } c;
+    c.h = __builtin_convertvector(x, half2_t);
+    return c.u;
+  } else {
+    union { bf162_t h; uint32_t u; } c;
+    c.h = __builtin_convertvector(x, bf162_t);
+    return c.u;
+  }
+}
+
+constexpr int kGqaTile = 32;             // tokens per wave step
+constexpr int kPRow = kGqaTile + 8;      // P^T row in LDS: 32 tokens + 16 bytes of padding
+
+// Registers of one 32-token step: K as 2 token groups x 4 dim steps, V as 8 dim blocks.
+struct GqaTile {
+  u32x4_t k[2][4];
+  u32x4_t v[8];
+};
+
+template <typename T, int BS, int G, int NW>
+__global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const DecodeParams P) {
+  using Geo = Geometry<BS>;
+  static_assert(G >= 2 && G <= 16, "group size");
+  // bf16 keeps 8 bits of a probability; P is carried as hi + lo parts then.
+  constexpr int kParts = __is_same(T, BF16) ? 2 : 1;
+  constexpr int kStep = kGqaTile * NW;   // wave w takes tokens t0 + 32 w + kStep n .. +31
+  __shared__ __attribute__((aligned(16))) uint16_t p_lds[NW][kParts][16][kPRow];
+  __shared__ __attribute__((aligned(16))) float x_acc[NW][G][kHeadSize];
+  __shared__ float x_ml[NW][G][2];
+  __shared__ int arrival;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int w = blockIdx.x;
+  int ii = 0;
+#pragma unroll
+  for (int k = 1; k < MUXA_MAX_DECODE_ITEMS; ++k)
+    if (k < P.n_items && w >= P.it[k].work_begin) ii = k;
+  const DecodeItemDev &I = P.it[ii];
+
+  const int WH = I.Hq / G;
+  const int local = w - I.work_begin;
+  const int e = local / WH;
+  Unit u;
+  u.item = ii;
+  u.wh = local - e * WH;
+  const int partition = P.partition;
+  if (!locate_pair_global(I.ctx, I.B, I.max_ctx, partition, e, lane, u.seq, u.split, u.ctx)) return;
+  u.t0 = u.split * partition;
+  u.t1 = min(u.ctx, u.t0 + partition);
+  const int hq0 = u.wh * G;
+  const int hk = hq0 / I.ratio;
+  const int t1 = u.t1;
+
+  const int h = lane & 15;               // this lane's head (columns >= G are padding)
+  const int g = lane >> 4;               // which 8 of an operand's 32 k-slots
+
+  // Q^T operand: dims 32 s + 8 g .. +7 of head h.
+  Frag8 qf[4];
+  {
+    const uint16_t *qrow = static_cast<const uint16_t *>(I.q) + static_cast<int64_t>(u.seq) * I.q_stride +
+                           (hq0 + (h < G ? h : 0)) * kHeadSize + 8 * g;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      // q rows are only 4-byte aligned in general.
+      const uint32_t *qp = reinterpret_cast<const uint32_t *>(qrow + 32 * s);
+      qf[s].u = h < G ? u32x4_t{qp[0], qp[1], qp[2], qp[3]} : u32x4_t{0, 0, 0, 0};
+    }
+  }
+
+  const int32_t *trow = I.tables + (static_cast<int64_t>(u.seq) * I.Hkv + hk) * I.max_blocks;
+  const u32x4_t *kpool = static_cast<const u32x4_t *>(P.k_pool);
+  const u32x4_t *vpool = static_cast<const u32x4_t *>(P.v_pool);
+  const int last_block = P.last_block;
+  const float scale_log2 = I.scale_log2;
+
+  v4f32_t oacc[8];                       // O^T[d = 16 nb + 4 g + i][head h]
+#pragma unroll
+  for (int nb = 0; nb < 8; ++nb) oacc[nb] = v4f32_t{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;          // running max (log2 units) and this lane's share of the sum
+
+  // Block ids of the step at tb: x, y for the K tokens tb + h and tb + 16 + h,
+  // z for the V tokens tb + 8 g .. +7 (0 past t1).  Clamped so that a corrupt
+  // table entry reads the wrong block instead of faulting the GPU.
+  auto load_ids = [&](int tb) {
+    int3 id = make_int3(0, 0, 0);
+    if (tb + h < t1) id.x = min(max(trow[(tb + h) / BS], 0), last_block);
+    if (tb + 16 + h < t1) id.y = min(max(trow[(tb + 16 + h) / BS], 0), last_block);
+    if (tb + 8 * g < t1) id.z = min(max(trow[(tb + 8 * g) / BS], 0), last_block);
+    return id;
+  };
+  auto issue = [&](GqaTile &r, int tb, int3 id) {
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg) {
+      const int tok = tb + 16 * tg + h;
+      const u32x4_t *kp = kpool + static_cast<int64_t>(tg ? id.y : id.x) * Geo::BLOCK_CHUNKS + (tok % BS);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) r.k[tg][s] = tok < t1 ? kp[(4 * s + g) * BS] : u32x4_t{0, 0, 0, 0};
+    }
+    const int tok = tb + 8 * g;
+    const u32x4_t *vp = vpool + static_cast<int64_t>(id.z) * Geo::BLOCK_CHUNKS + (tok % BS) / 8;
+#pragma unroll
+    for (int nb = 0; nb < 8; ++nb) r.v[nb] = tok < t1 ? vp[(16 * nb + h) * Geo::PARTS] : u32x4_t{0, 0, 0, 0};
+  };
+  auto compute = [&](GqaTile &r, int tb) {
+    const bool tail = tb + kGqaTile > t1;
+    if (tail) {
+      // Slots of tokens >= t1 were never written and may hold NaN/Inf patterns;
+      // their probability is 0 but 0 * NaN would still poison the product.
+      const int n_ok = t1 - (tb + 8 * g);
+#pragma unroll
+      for (int nb = 0; nb < 8; ++nb)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          if (2 * c >= n_ok) r.v[nb][c] = 0u;
+          else if (2 * c + 1 >= n_ok) r.v[nb][c] &= 0x0000ffffu;
+        }
+    }
+    // ---- S^T = K . Q^T ---------------------------------------------------------
+    v4f32_t sacc[2];
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg) {
+      sacc[tg] = v4f32_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        Frag8 kf;
+        kf.u = r.k[tg][s];
+        sacc[tg] = mfma16<T>(kf, qf[s], sacc[tg]);
+      }
+    }
+    // ---- online softmax: lane = head h, tokens tb + 16 tg + 4 g + i ----------------
+    float mx = -INFINITY;
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float sc = sacc[tg][i] * scale_log2;
+        if (tail && tb + 16 * tg + 4 * g + i >= t1) sc = -INFINITY;
+        sacc[tg][i] = sc;
+        mx = fmaxf(mx, sc);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));  // the step has at least one valid token: finite
+    const float m_new = fmaxf(m, mx);
+    const float alpha = fast_exp2(m - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg) {
+      float p[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        p[i] = fast_exp2(sacc[tg][i] - m_new);
+        psum += p[i];
+      }
+      const uint32_t w0 = pack_pair<T>(p[0], p[1]), w1 = pack_pair<T>(p[2], p[3]);
+      *reinterpret_cast<u32x2_t *>(&p_lds[wave][0][h][16 * tg + 4 * g]) = u32x2_t{w0, w1};
+      if constexpr (kParts == 2) {
+        const float r0 = p[0] - bf16_lo(w0), r1 = p[1] - bf16_hi(w0);
+        const float r2 = p[2] - bf16_lo(w1), r3 = p[3] - bf16_hi(w1);
+        *reinterpret_cast<u32x2_t *>(&p_lds[wave][1][h][16 * tg + 4 * g]) =
+            u32x2_t{pack_pair<T>(r0, r1), pack_pair<T>(r2, r3)};
+      }
+    }
+    l = l * alpha + psum;
+    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
+#pragma unroll
+      for (int nb = 0; nb < 8; ++nb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) oacc[nb][i] *= alpha;
+    }
+    m = m_new;
+    wave_lds_sync();
+    Frag8 pf[kParts];
+#pragma unroll
+    for (int part = 0; part < kParts; ++part)
+      pf[part].u = *reinterpret_cast<const u32x4_t *>(&p_lds[wave][part][h][8 * g]);
+    wave_lds_sync();
+    // ---- O^T += V^T . P^T --------------------------------------------------------
+#pragma unroll
+    for (int nb = 0; nb < 8; ++nb) {
+      Frag8 vf;
+      vf.u = r.v[nb];
+#pragma unroll
+      for (int part = 0; part < kParts; ++part) oacc[nb] = mfma16<T>(vf, pf[part], oacc[nb]);
+    }
+  };
+
+  // Two register sets: the loads of the next step are in flight while the
+  // current one is consumed, and the block ids run one step further ahead.
+  int tb = u.t0 + kGqaTile * wave;
+  if (tb < t1) {
+    GqaTile ra, rb;
+    issue(ra, tb, load_ids(tb));
+    int3 ids_next = make_int3(0, 0, 0);
+    if (tb + kStep < t1) ids_next = load_ids(tb + kStep);
+    while (true) {
+      const bool has_b = tb + kStep < t1;
+      if (has_b) {
+        issue(rb, tb + kStep, ids_next);
+        if (tb + 2 * kStep < t1) ids_next = load_ids(tb + 2 * kStep);
+      }
+      compute(ra, tb);
+      if (!has_b) break;
+      tb += kStep;
+      const bool has_a = tb + kStep < t1;
+      if (has_a) {
+        issue(ra, tb + kStep, ids_next);
+        if (tb + 2 * kStep < t1) ids_next = load_ids(tb + 2 * kStep);
+      }
+      compute(rb, tb);
+      if (!has_a) break;
+      tb += kStep;
+    }
+  }
+
+  // ---- this wave's partial to LDS, in the layout the merge expects ----------------------
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+  if (h < G) {
+#pragma unroll
+    for (int nb = 0; nb < 8; ++nb)
+      *reinterpret_cast<float4 *>(&x_acc[wave][h][16 * nb + 4 * g]) =
+          make_float4(oacc[nb][0], oacc[nb][1], oacc[nb][2], oacc[nb][3]);
+    if (g == 0) {
+      x_ml[wave][h][0] = m;
+      x_ml[wave][h][1] = l;
+    }
+  }
+  __syncthreads();
+  merge_and_write_group<T, G, NW>(I, u, partition, x_acc, x_ml, &arrival, lane, wave);
+}
+
 // Zero-fills the arrival counters (a kernel rather than a memset node so the
 // call can be captured into a graph).
 __global__ void fill_zero_kernel(int32_t *p, int64_t n) {
@@ -489,6 +855,7 @@ int choose_partition(const MuxDecodeItem *items, int n_items, int requested) {
 
 int pick_group(int ratio) {
   if (ratio == 8 || ratio == 4 || ratio == 2) return ratio;
+  if (ratio % 16 == 0) return 16;
   if (ratio % 8 == 0) return 8;
   if (ratio % 4 == 0) return 4;
   if (ratio % 2 == 0) return 2;
@@ -547,13 +914,21 @@ hipError_t launch_g(const DecodeParams &P, int grid, hipStream_t st) {
   return hipGetLastError();
 }
 
+template <typename T, int BS, int G>
+hipError_t launch_gqa(const DecodeParams &P, int grid, hipStream_t st) {
+  constexpr int NW = kWavesPerGroup;
+  hipLaunchKernelGGL((paged_decode_gqa_kernel<T, BS, G, NW>), dim3(grid), dim3(64 * NW), 0, st, P);
+  return hipGetLastError();
+}
+
 template <typename T, int BS>
 hipError_t launch_main(int G, const DecodeParams &P, int grid, hipStream_t st) {
   switch (G) {
     case 1: return launch_g<T, BS, 1>(P, grid, st);
     case 2: return launch_g<T, BS, 2>(P, grid, st);
-    case 4: return launch_g<T, BS, 4>(P, grid, st);
-    case 8: return launch_g<T, BS, 8>(P, grid, st);
+    case 4: return launch_gqa<T, BS, 4>(P, grid, st);
+    case 8: return launch_gqa<T, BS, 8>(P, grid, st);
+    case 16: return launch_gqa<T, BS, 16>(P, grid, st);
     default: return hipErrorInvalidValue;
   }
 }

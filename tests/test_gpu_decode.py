@@ -194,12 +194,31 @@ def test_decode_other_block_sizes(bs):
     _check(got, want)
 
 
-@pytest.mark.parametrize("Hq,Hkv", [(8, 4), (8, 2), (16, 2), (6, 2), (64, 8)])
+@pytest.mark.parametrize("Hq,Hkv", [(8, 4), (8, 2), (16, 2), (6, 2), (64, 8), (32, 2), (32, 1)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_decode_gqa(Hq, Hkv, dtype):
     _announce(f"decode gqa Hq={Hq} Hkv={Hkv} {dtype}")
     got, want = _decode_case(5, [5, 64, 130, 700], Hq, Hkv, 16, dtype=dtype, partition=256)
     _check(got, want, out_dtype=dtype)
+
+
+@pytest.mark.parametrize("bs", [8, 32])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_decode_gqa_other_block_sizes(bs, dtype):
+    """The matrix-core path (4 or more query heads per kv head) at every block size,
+    with contexts around the block, tile and partition boundaries."""
+    _announce(f"decode gqa bs={bs} {dtype}")
+    got, want = _decode_case(8, [1, 7, 8, 9, 31, 32, 33, 63, 64, 65, 100, 128, 129, 400], 8, 2, bs,
+                             dtype=dtype, partition=128, repeat=2)
+    _check(got, want, out_dtype=dtype)
+
+
+def test_decode_gqa_short_contexts_keep_probability_precision():
+    """One to three keys: probabilities near 1 must not lose mantissa bits on
+    their way into the P.V product (bf16 carries them as hi + lo parts)."""
+    _announce("decode gqa short contexts bf16")
+    got, want = _decode_case(11, [1, 2, 3, 2, 1, 3], 16, 2, 16, dtype=torch.bfloat16)
+    _check(got, want, out_dtype=torch.bfloat16)
 
 
 def test_decode_layer_slice_and_strided_q():
