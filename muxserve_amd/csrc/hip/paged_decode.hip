@@ -846,11 +846,23 @@ __global__ void fill_zero_kernel(int32_t *p, int64_t n) {
 // ---------------------------------------------------------------------------
 namespace {
 
+int pick_group(int ratio);
+
+// Tokens per partition when the caller leaves the choice to the library: short
+// partitions spread the batch over more workgroups, long ones amortise a unit's
+// fixed cost; the grouped-query kernel streams a partition with its loads
+// overlapped and prefers the longer ones.
 int choose_partition(const MuxDecodeItem *items, int n_items, int requested) {
   if (requested > 0) return requested;
   int max_ctx = 0;
-  for (int i = 0; i < n_items; ++i) max_ctx = std::max(max_ctx, items[i].max_context_len);
-  return max_ctx > 4096 ? 512 : 256;
+  bool all_grouped = true;
+  for (int i = 0; i < n_items; ++i) {
+    max_ctx = std::max(max_ctx, items[i].max_context_len);
+    if (items[i].num_kv_heads <= 0 || pick_group(items[i].num_q_heads / items[i].num_kv_heads) < 4)
+      all_grouped = false;
+  }
+  if (max_ctx <= 4096) return 256;
+  return all_grouped ? 1024 : 512;
 }
 
 int pick_group(int ratio) {

@@ -115,6 +115,50 @@ def test_reshape_and_cache_bit_exact_random_slots(bs, dtype):
     assert torch.equal(dv.cpu().view(torch.int16), v_pool.view(torch.int16))
 
 
+@pytest.mark.parametrize("bs", [16, 8, 32])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_reshape_and_cache_bit_exact_runs_of_consecutive_slots(bs, dtype):
+    """Runs of consecutive slots take the 16-byte V store path when 8 tokens
+    that the kernel groups together start a pool chunk; every way of almost
+    qualifying (misaligned start, a skipped token inside, a run broken in the
+    middle, a run cut by the end of the batch, reversed order) must fall back
+    to the element path and still match the oracle bitwise."""
+    _announce(f"reshape_and_cache slot runs bs={bs} {dtype}")
+    g = torch.Generator().manual_seed(100 + bs)
+    L, H, layer, N = 2, 3, 1, 64
+    per_head = []
+    for h in range(H):
+        base = (h * 20 + 1) * bs                       # block-aligned, blocks disjoint between heads
+        col = np.concatenate([
+            base + np.arange(16),                      # tokens 0-15: two aligned chunks
+            base + 16 + 3 + np.arange(8),              # 16-23: consecutive but misaligned start
+            base + 32 + np.arange(8),                  # 24-31: aligned ...
+            base + 48 + np.arange(8)[::-1],            # 32-39: right slots, reversed order
+            base + 64 + np.arange(8),                  # 40-47: aligned, one token skipped below
+            base + 80 + np.array([0, 1, 2, 3, 12, 13, 14, 15]),   # 48-55: broken in the middle
+            base + 96 + np.arange(5),                  # 56-60: run cut by the end of the batch
+        ]).astype(np.int64)
+        per_head.append(col)
+    T = len(per_head[0])
+    slots = np.full((T, L, H), -1, dtype=np.int64)
+    for h in range(H):
+        slots[:, layer, h] = per_head[h]
+    slots[43, layer, 1] = -1
+    slots[:, 0, :] = 7                                 # another layer's column must be ignored
+    pad = (T + 7) // 8 * 8
+    k = torch.randn((pad, H * HEAD_SIZE), generator=g).to(dtype)
+    v = torch.randn((pad, H * HEAD_SIZE), generator=g).to(dtype)
+    k_pool, v_pool = orc.allocate_pool(N, bs, dtype)
+    k_pool.copy_(torch.randn(k_pool.shape, generator=g).to(dtype))
+    v_pool.copy_(torch.randn(v_pool.shape, generator=g).to(dtype))
+    dk, dv = k_pool.to(DEV), v_pool.to(DEV)
+    ops.reshape_and_cache(k.to(DEV), v.to(DEV), dk, dv, torch.from_numpy(slots).to(DEV), layer=layer, num_tokens=T)
+    torch.cuda.synchronize()
+    orc.reshape_and_cache(k, v, k_pool, v_pool, torch.from_numpy(slots), layer=layer, num_tokens=T)
+    assert torch.equal(dk.cpu().view(torch.int16), k_pool.view(torch.int16))
+    assert torch.equal(dv.cpu().view(torch.int16), v_pool.view(torch.int16))
+
+
 def test_reshape_and_cache_prefill_pattern_roundtrip():
     """Prompt-shaped slots (token i -> block i//bs, offset i%bs per head), then
     gather back through the tables: gather(scatter(x)) == x bitwise."""
