@@ -51,6 +51,7 @@ struct DecodeItemDev {
   float *ws_acc;                  // [B, Hq, max_splits, 128]
   float *ws_ml;                   // [B, Hq, max_splits, 2]  (running max in log2 units, sum)
   int32_t *counters;              // [B, Hq/G] arrivals per (sequence, head group); zero between launches
+  const int4 *unit_table;         // large batches: (sequence, partition index, ctx, -) per pair, else null
   int32_t B, Hq, Hkv, ratio;      // ratio = Hq / Hkv
   int32_t max_blocks, max_splits, max_ctx;
   int32_t work_begin;             // first block of this item in the grid
@@ -421,62 +422,153 @@ __device__ __forceinline__ void merge_and_write_group(const DecodeItemDev &I, co
 //   2. all full partitions of those sequences;
 //   3. sequences that fit one partition (ctx <= partition): no partials, no
 //      atomics, the output is written straight from the workgroup.
-__device__ __forceinline__ bool locate_pair_global(const int32_t *ctx_arr, int B, int max_ctx, int partition,
-                                                   int e, int lane, int &seq, int &split, int &ctx) {
+
+// Lane index of the n-th (0-based) set bit of a wave mask that has more than n bits set.
+__device__ __forceinline__ int nth_set_lane(unsigned long long mask, int n, int lane) {
+  const int upto = __popcll(mask & (~0ull >> (63 - lane)));          // set bits in lanes 0..lane
+  const unsigned long long hit = __builtin_amdgcn_ballot_w64(((mask >> lane) & 1ull) != 0 && upto == n + 1);
+  return __ffsll(static_cast<long long>(hit)) - 1;
+}
+
+// Batches of at most 64 * kLocateChunks sequences: all context lengths are
+// fetched with one round of loads (lane l keeps sequences l, l+64, ...) and the
+// three classes are enumerated from registers, so the unit is known after a
+// single memory latency.
+constexpr int kLocateChunks = 4;
+__device__ __forceinline__ bool locate_pair_small(const int32_t *ctx_arr, int B, int max_ctx, int partition,
+                                                  int e, int lane, int &seq, int &split, int &ctx) {
+  int c[kLocateChunks], full[kLocateChunks];
+#pragma unroll
+  for (int j = 0; j < kLocateChunks; ++j) {
+    const int s = 64 * j + lane;
+    c[j] = s < B ? ctx_arr[s] : 0;
+  }
+  unsigned long long rem_mask[kLocateChunks];
+#pragma unroll
+  for (int j = 0; j < kLocateChunks; ++j) {
+    c[j] = max(min(c[j], max_ctx), 0);
+    const int q = c[j] / partition;
+    full[j] = c[j] > partition ? q : 0;
+    rem_mask[j] = __builtin_amdgcn_ballot_w64(c[j] > partition && c[j] != q * partition);
+  }
   int base = 0;
   // class 1: remainders of split sequences
-  for (int c0 = 0; c0 < B; c0 += 64) {
-    const int s = c0 + lane;
-    const int c = s < B ? max(min(ctx_arr[s], max_ctx), 0) : 0;
-    const bool hit_class = c > partition && (c % partition) != 0;
-    const unsigned long long mask = __builtin_amdgcn_ballot_w64(hit_class);
-    const int cnt = __popcll(mask);
+#pragma unroll
+  for (int j = 0; j < kLocateChunks; ++j) {
+    const int cnt = __popcll(rem_mask[j]);
     if (e < base + cnt) {
-      const int upto = __popcll(mask & (~0ull >> (63 - lane)));     // class members in lanes 0..lane
-      const unsigned long long hit = __builtin_amdgcn_ballot_w64(hit_class && upto == e - base + 1);
-      const int k = __ffsll(static_cast<long long>(hit)) - 1;
-      seq = c0 + k;
-      ctx = __builtin_amdgcn_readlane(c, k);
+      const int k = nth_set_lane(rem_mask[j], e - base, lane);
+      seq = 64 * j + k;
+      ctx = __builtin_amdgcn_readlane(c[j], k);
       split = ctx / partition;
       return true;
     }
     base += cnt;
   }
   // class 2: full partitions of split sequences
-  for (int c0 = 0; c0 < B; c0 += 64) {
-    const int s = c0 + lane;
-    const int c = s < B ? max(min(ctx_arr[s], max_ctx), 0) : 0;
-    const int full = c > partition ? c / partition : 0;
-    const int incl = wave_inclusive_scan(full);
+#pragma unroll
+  for (int j = 0; j < kLocateChunks; ++j) {
+    const int incl = wave_inclusive_scan(full[j]);
     const int total = __builtin_amdgcn_readlane(incl, 63);
     if (e < base + total) {
       const int k = __popcll(__builtin_amdgcn_ballot_w64(base + incl <= e));
-      seq = c0 + k;
-      split = e - base - __builtin_amdgcn_readlane(incl - full, k);
-      ctx = __builtin_amdgcn_readlane(c, k);
+      seq = 64 * j + k;
+      split = e - base - __builtin_amdgcn_readlane(incl - full[j], k);
+      ctx = __builtin_amdgcn_readlane(c[j], k);
       return true;
     }
     base += total;
   }
   // class 3: sequences that fit one partition
-  for (int c0 = 0; c0 < B; c0 += 64) {
-    const int s = c0 + lane;
-    const int c = s < B ? max(min(ctx_arr[s], max_ctx), 0) : 0;
-    const bool hit_class = c > 0 && c <= partition;
-    const unsigned long long mask = __builtin_amdgcn_ballot_w64(hit_class);
+#pragma unroll
+  for (int j = 0; j < kLocateChunks; ++j) {
+    const unsigned long long mask = __builtin_amdgcn_ballot_w64(c[j] > 0 && c[j] <= partition);
     const int cnt = __popcll(mask);
     if (e < base + cnt) {
-      const int upto = __popcll(mask & (~0ull >> (63 - lane)));
-      const unsigned long long hit = __builtin_amdgcn_ballot_w64(hit_class && upto == e - base + 1);
-      const int k = __ffsll(static_cast<long long>(hit)) - 1;
-      seq = c0 + k;
-      ctx = __builtin_amdgcn_readlane(c, k);
+      const int k = nth_set_lane(mask, e - base, lane);
+      seq = 64 * j + k;
+      ctx = __builtin_amdgcn_readlane(c[j], k);
       split = 0;
       return true;
     }
     base += cnt;
   }
   return false;
+}
+
+// Batches too large for that take the pair from a table that a small kernel
+// (decode_plan_kernel below) writes ahead of the launch: one 16-byte load.
+__device__ __forceinline__ bool locate_pair(const DecodeItemDev &I, int partition, int e, int lane, int &seq,
+                                            int &split, int &ctx) {
+  if (I.unit_table == nullptr) return locate_pair_small(I.ctx, I.B, I.max_ctx, partition, e, lane, seq, split, ctx);
+  const int4 ent = I.unit_table[e];
+  if (ent.x < 0) return false;
+  seq = ent.x;
+  split = ent.y;
+  ctx = ent.z;
+  return true;
+}
+
+// Writes the (sequence, partition) table of one item per workgroup, in the same
+// three classes as above.  Thread t owns a contiguous range of sequences;
+// class counts are prefix-summed over the threads in LDS.  Entries past the
+// last pair (the grid is sized from an upper bound) get sequence -1.
+struct PlanItem {
+  const int32_t *ctx;
+  int4 *table;
+  int32_t B, max_ctx, capacity;   // capacity = entries in table
+};
+struct PlanParams {
+  PlanItem it[MUXA_MAX_DECODE_ITEMS];
+  int32_t partition;
+};
+
+__global__ __launch_bounds__(256) void decode_plan_kernel(const PlanParams PP) {
+  __shared__ int scan[3][256];
+  const PlanItem &I = PP.it[blockIdx.x];
+  const int partition = PP.partition;
+  const int t = threadIdx.x;
+  const int per = (I.B + 255) / 256;
+  const int s0 = min(t * per, I.B), s1 = min(s0 + per, I.B);
+  int n[3] = {0, 0, 0};
+  for (int s = s0; s < s1; ++s) {
+    const int c = max(min(I.ctx[s], I.max_ctx), 0);
+    const int q = c / partition;
+    if (c > partition) {
+      n[1] += q;
+      if (c != q * partition) n[0] += 1;
+    } else if (c > 0) {
+      n[2] += 1;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 3; ++k) scan[k][t] = n[k];
+  __syncthreads();
+  for (int d = 1; d < 256; d <<= 1) {      // inclusive Hillis-Steele scan of the three rows
+    int v[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) v[k] = t >= d ? scan[k][t - d] : 0;
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 3; ++k) scan[k][t] += v[k];
+    __syncthreads();
+  }
+  const int tot0 = scan[0][255], tot1 = scan[1][255], tot2 = scan[2][255];
+  int at0 = scan[0][t] - n[0];
+  int at1 = tot0 + scan[1][t] - n[1];
+  int at2 = tot0 + tot1 + scan[2][t] - n[2];
+  for (int s = s0; s < s1; ++s) {
+    const int c = max(min(I.ctx[s], I.max_ctx), 0);
+    const int q = c / partition;
+    if (c > partition) {
+      for (int j = 0; j < q; ++j)
+        if (at1 < I.capacity) I.table[at1++] = make_int4(s, j, c, 0);
+      if (c != q * partition && at0 < I.capacity) I.table[at0++] = make_int4(s, q, c, 0);
+    } else if (c > 0) {
+      if (at2 < I.capacity) I.table[at2++] = make_int4(s, 0, c, 0);
+    }
+  }
+  for (int i = tot0 + tot1 + tot2 + t; i < I.capacity; i += 256) I.table[i] = make_int4(-1, 0, 0, 0);
 }
 
 // q of the unit's head group for the tile code.  G == 1: one coalesced 256-byte
@@ -513,7 +605,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_kernel(const DecodeParam
 #pragma unroll
   for (int k = 1; k < MUXA_MAX_DECODE_ITEMS; ++k)
     if (k < P.n_items && w >= P.it[k].work_begin) ii = k;
-  const DecodeItemDev &I = P.it[ii];
+  const DecodeItemDev I = P.it[ii];       // by value: one round of scalar loads for every field
 
   const int WH = I.Hq / G;                   // head groups per sequence
   const int local = w - I.work_begin;
@@ -523,18 +615,21 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_kernel(const DecodeParam
   u.wh = local - e * WH;
   const int partition = P.partition;
   // Every wave of the workgroup derives the same unit (or all of them leave).
-  if (!locate_pair_global(I.ctx, I.B, I.max_ctx, partition, e, lane, u.seq, u.split, u.ctx)) return;
+  if (!locate_pair(I, partition, e, lane, u.seq, u.split, u.ctx)) return;
   u.t0 = u.split * partition;
   u.t1 = min(u.ctx, u.t0 + partition);
   const int hq0 = u.wh * G;
   const int hk = hq0 / I.ratio;
 
-  uint32_t q_s[64];
-  fetch_q<G>(I, u.seq, hq0, lane, q_s, q_lds[wave]);
-
+  // The first tile's block ids and q are independent: both loads are issued
+  // before either is waited for.
   const int32_t *trow = I.tables + (static_cast<int64_t>(u.seq) * I.Hkv + hk) * I.max_blocks;
   const uint4 *kpool = static_cast<const uint4 *>(P.k_pool);
   const uint4 *vpool = static_cast<const uint4 *>(P.v_pool);
+  const int tb0 = u.t0 + wave * 64;
+  int id_next = load_block_id<BS>(trow, tb0, u.t1, lane, P.last_block);
+  uint32_t q_s[64];
+  fetch_q<G>(I, u.seq, hq0, lane, q_s, q_lds[wave]);
 
   float m[G], l[G], acc[G][Geo::VI];
 #pragma unroll
@@ -544,8 +639,9 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_kernel(const DecodeParam
 #pragma unroll
     for (int j = 0; j < Geo::VI; ++j) acc[g][j] = 0.f;
   }
-  for (int tb = u.t0 + wave * 64; tb < u.t1; tb += 64 * NW) {
-    const int id = load_block_id<BS>(trow, tb, u.t1, lane, P.last_block);
+  for (int tb = tb0; tb < u.t1; tb += 64 * NW) {
+    const int id = id_next;
+    if (tb + 64 * NW < u.t1) id_next = load_block_id<BS>(trow, tb + 64 * NW, u.t1, lane, P.last_block);
     uint4 kreg[16];
     uint4 vreg[Geo::BPT][Geo::VI];
     issue_tile_loads<BS>(kreg, vreg, kpool, vpool, id, tb, u.t1, lane);
@@ -640,7 +736,7 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
 #pragma unroll
   for (int k = 1; k < MUXA_MAX_DECODE_ITEMS; ++k)
     if (k < P.n_items && w >= P.it[k].work_begin) ii = k;
-  const DecodeItemDev &I = P.it[ii];
+  const DecodeItemDev I = P.it[ii];       // by value: one round of scalar loads for every field
 
   const int WH = I.Hq / G;
   const int local = w - I.work_begin;
@@ -649,7 +745,7 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
   u.item = ii;
   u.wh = local - e * WH;
   const int partition = P.partition;
-  if (!locate_pair_global(I.ctx, I.B, I.max_ctx, partition, e, lane, u.seq, u.split, u.ctx)) return;
+  if (!locate_pair(I, partition, e, lane, u.seq, u.split, u.ctx)) return;
   u.t0 = u.split * partition;
   u.t1 = min(u.ctx, u.t0 + partition);
   const int hq0 = u.wh * G;
@@ -878,22 +974,25 @@ struct ItemPlan {
   size_t counters_off, acc_off, ml_off;
   int max_splits;
   int64_t units;      // (sequence, partition) pairs reserved in the direct kernel's grid
+  size_t table_off;   // pair table of a large batch (0: none)
 };
 
 // Workspace layout: a FIXED leading region of MUXA_DECODE_COUNTER_BYTES holds
 // the arrival counters (one int32 per sequence and head group, items back to
 // back) so that its position never depends on the shapes of a call and no
 // call's partials can land on another call's counters; then per item acc
-// [B,Hq,max_splits,128] fp32 and ml [B,Hq,max_splits,2] fp32.  Calls whose
-// contexts all fit one partition need no workspace.  Returns total bytes, or
-// SIZE_MAX when the counters do not fit the fixed region.
+// [B,Hq,max_splits,128] fp32 and ml [B,Hq,max_splits,2] fp32, and for batches
+// of more than 64 * kLocateChunks sequences the pair table (16 bytes per pair).
+// Calls whose contexts all fit one partition and whose batches are small need no
+// workspace.  Returns total bytes, or SIZE_MAX when the counters do not fit the
+// fixed region.
 size_t plan_workspace(const MuxDecodeItem *items, int n_items, int partition, ItemPlan *out) {
   size_t counters = 0;
   size_t off = MUXA_DECODE_COUNTER_BYTES;
   bool any = false;
   for (int i = 0; i < n_items; ++i) {
     const MuxDecodeItem &it = items[i];
-    ItemPlan w{0, 0, 0, std::max(1, (it.max_context_len + partition - 1) / partition), 0};
+    ItemPlan w{0, 0, 0, std::max(1, (it.max_context_len + partition - 1) / partition), 0, 0};
     // Upper bound on the number of pairs: every sequence has at most
     // max_splits of them, and all sequences together at most
     // floor(sum ctx / partition) full ones plus one remainder each.
@@ -910,6 +1009,12 @@ size_t plan_workspace(const MuxDecodeItem *items, int n_items, int partition, It
       off += rows * kHeadSize * sizeof(float);
       w.ml_off = off;
       off += rows * 2 * sizeof(float);
+      off = (off + 255) & ~static_cast<size_t>(255);
+    }
+    if (it.num_seqs > 64 * kLocateChunks && it.max_context_len > 0) {
+      any = true;
+      w.table_off = off;
+      off += static_cast<size_t>(w.units) * sizeof(int4);
       off = (off + 255) & ~static_cast<size_t>(255);
     }
     if (out) out[i] = w;
@@ -1031,6 +1136,9 @@ int32_t mux_multi_decode(const MuxDecodeItem *items, int32_t n_items,
     if (done[first]) continue;
     const int G = pick_group(items[first].num_q_heads / items[first].num_kv_heads);
     DecodeParams P;
+    PlanParams PP;
+    PP.partition = partition;
+    int n_tables = 0;
     P.k_pool = k_pool;
     P.v_pool = v_pool;
     P.partition = partition;
@@ -1055,6 +1163,17 @@ int32_t mux_multi_decode(const MuxDecodeItem *items, int32_t n_items,
       d.ws_acc = split ? reinterpret_cast<float *>(ws + plan[i].acc_off) : nullptr;
       d.ws_ml = split ? reinterpret_cast<float *>(ws + plan[i].ml_off) : nullptr;
       d.counters = split ? reinterpret_cast<int32_t *>(ws + plan[i].counters_off) : nullptr;
+      d.unit_table = nullptr;
+      if (plan[i].table_off != 0) {
+        if (plan[i].units > 0x7fffffff) return MUXA_EUNSUPPORTED;
+        PlanItem &t = PP.it[n_tables++];
+        t.ctx = it.context_lens;
+        t.table = reinterpret_cast<int4 *>(ws + plan[i].table_off);
+        t.B = it.num_seqs;
+        t.max_ctx = it.max_context_len;
+        t.capacity = static_cast<int32_t>(plan[i].units);
+        d.unit_table = t.table;
+      }
       d.B = it.num_seqs;
       d.Hq = it.num_q_heads;
       d.Hkv = it.num_kv_heads;
@@ -1068,6 +1187,11 @@ int32_t mux_multi_decode(const MuxDecodeItem *items, int32_t n_items,
       if (work > 0x7fffffff) return MUXA_EUNSUPPORTED;
     }
     if (P.n_items == 0) continue;
+    if (n_tables > 0) {
+      hipLaunchKernelGGL(decode_plan_kernel, dim3(n_tables), dim3(256), 0, st, PP);
+      hipError_t pe = hipGetLastError();
+      if (pe != hipSuccess) return hip_fail(pe);
+    }
     const int grid = static_cast<int>(work);
     hipError_t e = dtype == MUXA_DTYPE_F16 ? launch_bs<F16>(block_size, G, P, grid, st)
                                            : launch_bs<BF16>(block_size, G, P, grid, st);

@@ -218,10 +218,11 @@ def test_decode_split_context_equals_single_pass(partition):
     _check(got, want)
 
 
-@pytest.mark.parametrize("B", [65, 130])
+@pytest.mark.parametrize("B", [65, 130, 300])
 @pytest.mark.parametrize("hint", [False, True])
 def test_decode_more_sequences_than_a_wave(B, hint):
-    """Unit enumeration walks the context lengths 64 sequences at a time."""
+    """Unit enumeration keeps up to 256 context lengths in registers and walks
+    larger batches 64 sequences at a time."""
     _announce(f"decode B={B} hint={hint}")
     rng = np.random.Generator(np.random.PCG64(B))
     ctx = rng.integers(1, 400, size=B)
