@@ -62,6 +62,36 @@ def test_prefill_matches_oracle_ragged_prompts(Hq, Hkv, dtype):
     assert excess <= 0, f"max-abs error {(got - want).abs().max().item():.3e}"
 
 
+@pytest.mark.parametrize("num_prompts", [64, 70, 150])
+def test_prefill_many_prompts_ties_and_empty_prompts(num_prompts):
+    """Many prompts in one launch: equal lengths, empty prompts and lengths
+    around the 128-row tile all appear."""
+    _announce(f"prefill {num_prompts} prompts")
+    rng = np.random.Generator(np.random.PCG64(num_prompts))
+    lens = rng.integers(1, 200, size=num_prompts)
+    lens[::5] = 128
+    lens[1::9] = 129
+    lens[3] = 0
+    lens[num_prompts - 2] = 0
+    lens[7] = 260
+    lens = [int(n) for n in lens]
+    got, q, k, v = _run_prefill(3, lens, 2, 1, torch.float16)
+    want = orc.prefill_causal(q, k, v, lens, D ** -0.5, 1)
+    assert torch.isfinite(got).all()
+    excess = ((got - want).abs() - _bound(want, torch.float16)).max().item()
+    assert excess <= 0, f"max-abs error {(got - want).abs().max().item():.3e}"
+
+
+@pytest.mark.parametrize("Hkv", [5, 9, 13])
+def test_prefill_kv_head_counts_that_do_not_divide_by_eight(Hkv):
+    _announce(f"prefill Hkv={Hkv}")
+    lens = [130, 17, 64]
+    got, q, k, v = _run_prefill(4, lens, Hkv, Hkv, torch.float16)
+    want = orc.prefill_causal(q, k, v, lens, D ** -0.5, Hkv)
+    excess = ((got - want).abs() - _bound(want, torch.float16)).max().item()
+    assert excess <= 0, f"max-abs error {(got - want).abs().max().item():.3e}"
+
+
 def test_prefill_long_prompt_and_unstrided_inputs():
     _announce("prefill long prompt")
     lens = [2048, 5, 700]
