@@ -159,6 +159,34 @@ def test_reshape_and_cache_bit_exact_runs_of_consecutive_slots(bs, dtype):
     assert torch.equal(dv.cpu().view(torch.int16), v_pool.view(torch.int16))
 
 
+@pytest.mark.parametrize("bs", [16, 8, 32])
+def test_reshape_and_cache_bit_exact_packed_ragged_prompts(bs):
+    """Prompts of every length 1..40 packed back to back: slot runs begin at
+    every phase of the kernel's 16-token grid and end in partial chunks."""
+    _announce(f"reshape_and_cache packed ragged prompts bs={bs}")
+    rng = np.random.Generator(np.random.PCG64(200 + bs))
+    g = torch.Generator().manual_seed(200 + bs)
+    H = 3
+    lens = rng.permutation(np.arange(1, 41)).astype(np.int32)
+    T = int(lens.sum())
+    N = int(((lens + bs - 1) // bs).sum()) * H + 9
+    ids = rng.permutation(N)
+    slots, used = workloads.prefill_slot_mapping(lens, H, bs, ids)
+    assert slots.shape == (T, 1, H)
+    pad = (T + 7) // 8 * 8
+    k = torch.randn((pad, H * HEAD_SIZE), generator=g).half()
+    v = torch.randn((pad, H * HEAD_SIZE), generator=g).half()
+    k_pool, v_pool = orc.allocate_pool(N, bs, torch.float16)
+    k_pool.copy_(torch.randn(k_pool.shape, generator=g).half())
+    v_pool.copy_(torch.randn(v_pool.shape, generator=g).half())
+    dk, dv = k_pool.to(DEV), v_pool.to(DEV)
+    ops.reshape_and_cache(k.to(DEV), v.to(DEV), dk, dv, torch.from_numpy(slots).to(DEV), num_tokens=T)
+    torch.cuda.synchronize()
+    orc.reshape_and_cache(k, v, k_pool, v_pool, torch.from_numpy(slots), num_tokens=T)
+    assert torch.equal(dk.cpu().view(torch.int16), k_pool.view(torch.int16))
+    assert torch.equal(dv.cpu().view(torch.int16), v_pool.view(torch.int16))
+
+
 def test_reshape_and_cache_prefill_pattern_roundtrip():
     """Prompt-shaped slots (token i -> block i//bs, offset i%bs per head), then
     gather back through the tables: gather(scatter(x)) == x bitwise."""
