@@ -34,6 +34,11 @@ HBM_PEAK_GBS = 8000.0
 # from the FETCH_SIZE / WRITE_SIZE counter passes summarised in
 # profiles/paged_decode_mixed3_hbm_traffic.txt (421.0 MB measured / 410.6 MB).
 MIXED3_TRAFFIC_RATIO = 1.025
+# Same for the grouped-query decode kernel (profiles/paged_decode_gqa_long_kernel_trace_and_traffic.txt:
+# 1394.5 MB / 1358.8 MB) and the prefill-shaped cache write (profiles/other_kernels_kernel_trace.txt:
+# 224.0 MB / 219.8 MB).
+GQA_LONG_TRAFFIC_RATIO = 1.026
+CACHE_WRITE_TRAFFIC_RATIO = 1.019
 
 
 def parse():
@@ -205,7 +210,9 @@ def bench_cache_write(args):
            "decode_shape": "7b/13b/30b, 56 tokens, three launches", "decode_ms": ms_d, "decode_bytes": bytes_d,
            "decode_gbs": bytes_d / (ms_d * 1e-3) / 1e9}
     roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-            "traffic": None, "kernel": "reshape_and_cache_kernel"}
+            "traffic": bytes_p * CACHE_WRITE_TRAFFIC_RATIO,
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiles/other_kernels_kernel_trace.txt",
+            "kernel": "reshape_and_cache_kernel"}
     return _line("KV-cache write tokens/s (prefill-shaped, 52 heads)", T / (ms_p * 1e-3), "tokens/s", args, ms_p,
                  cfg, roof, dtype="u16")
 
@@ -305,7 +312,10 @@ def bench_gqa_long(args):
     cfg = {"workload": "gqa_long", "shape": "Hq64/Hkv8, B=64, ctx U[2048,8192], bf16", "pool_gb": round(N * 8192 / 1e9, 1),
            "bytes_per_step": int(nbytes), "partition": args.partition}
     roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-            "traffic": None, "kernel": "paged_decode_gqa_kernel<BF16,16,8,4>"}
+            "traffic": nbytes * GQA_LONG_TRAFFIC_RATIO,
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+                              "profiles/paged_decode_gqa_long_kernel_trace_and_traffic.txt",
+            "kernel": "paged_decode_gqa_kernel<BF16,16,8,4>"}
     return _line("long-context GQA decode attn tokens/s", 64 / (ms * 1e-3), "tokens/s", args, ms, cfg, roof, dtype="bf16")
 
 

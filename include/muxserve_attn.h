@@ -92,7 +92,10 @@ int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t kv_row_strid
  * context_lens (the serving loop has them on the host before the copy,
  * llm_runtime.py:311-326); it only tightens the grid, 0 = unknown.
  * partition_size: tokens per split of a context (multiple of 64), 0 = choose.
- * workspace: scratch for split partials, at least
+ * workspace: scratch for the partial results of split contexts and, for
+ * batches of more than 256 sequences, the table that maps workgroups to
+ * (sequence, partition) pairs (written by a small kernel launched ahead of
+ * the attention kernel on the same stream); at least
  * mux_paged_decode_workspace_bytes(...) bytes, 16-byte aligned; may be NULL
  * when that is 0.  Its first MUXA_DECODE_COUNTER_BYTES bytes are arrival
  * counters that must be ZERO when a launch begins: zero them once with
