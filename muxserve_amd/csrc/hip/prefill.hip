@@ -192,6 +192,8 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
 
     // ---- S^T = K . Q^T : two 32-key blocks ------------------------------------------
     // LDS fragment reads run kDepth steps ahead of the MFMAs that consume them.
+    // Consecutive MFMAs go to different accumulators (2 key blocks here, 4 dim
+    // blocks in the P.V product): a single dependent chain runs at 3/4 of the rate.
     constexpr int kDepth = 4;
     v16f32 sacc[2];
 #pragma unroll
@@ -203,14 +205,14 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
       Frag ring[kDepth];
 #pragma unroll
       for (int j = 0; j < kDepth; ++j)
-        ring[j].u = *reinterpret_cast<const u32x4 *>(kr + (j / 8) * 32 * kKRow + 16 * (j % 8));
+        ring[j].u = *reinterpret_cast<const u32x4 *>(kr + (j % 2) * 32 * kKRow + 16 * (j / 2));
       __builtin_amdgcn_sched_barrier(0);   // keep the scheduler from sinking the reads to their uses
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
-        sacc[j / 8] = mfma<T>(ring[j % kDepth], qf[j % 8], sacc[j / 8]);
+        sacc[j % 2] = mfma<T>(ring[j % kDepth], qf[j / 2], sacc[j % 2]);
         if (j + kDepth < 16) {
           const int n = j + kDepth;
-          ring[j % kDepth].u = *reinterpret_cast<const u32x4 *>(kr + (n / 8) * 32 * kKRow + 16 * (n % 8));
+          ring[j % kDepth].u = *reinterpret_cast<const u32x4 *>(kr + (n % 2) * 32 * kKRow + 16 * (n / 2));
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -284,8 +286,8 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
     // k-slot j of lane half h in step (kb, st) is key 32 kb + 16 st + 8 (j/4) + 4 h + j%4
     {
       const uint16_t *vr = &Vt[qcol * kVRow + 4 * half];
-      auto read_v = [&](int n) {         // fragment n = 4 mb + ks
-        const uint16_t *r = vr + (n / 4) * 32 * kVRow + 16 * (n % 4);
+      auto read_v = [&](int n) {         // fragment n = 4 ks + mb
+        const uint16_t *r = vr + (n % 4) * 32 * kVRow + 16 * (n / 4);
         const u32x2 lo = *reinterpret_cast<const u32x2 *>(r);
         const u32x2 hi = *reinterpret_cast<const u32x2 *>(r + 8);
         Frag f;
@@ -298,8 +300,8 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
-        oacc[j / 4] = mfma<T>(ring[j % kDepth], pf[j % 4], oacc[j / 4]);
-        if constexpr (kSplitP) oacc[j / 4] = mfma<T>(ring[j % kDepth], pf_lo[j % 4], oacc[j / 4]);
+        oacc[j % 4] = mfma<T>(ring[j % kDepth], pf[j / 4], oacc[j % 4]);
+        if constexpr (kSplitP) oacc[j % 4] = mfma<T>(ring[j % kDepth], pf_lo[j / 4], oacc[j % 4]);
         if (j + kDepth < 16) ring[j % kDepth] = read_v(j + kDepth);
         __builtin_amdgcn_sched_barrier(0);
       }
