@@ -354,6 +354,42 @@ def test_multi_decode_three_models_one_launch_matches_separate_launches():
         _check(f[:m.batch].float().cpu(), want)
 
 
+def test_multi_decode_mixed_head_groupings_and_a_large_batch_share_one_workspace():
+    """One call with a grouped-query model (matrix-core kernel), a small
+    multi-head model (register lookup) and a 300-sequence multi-head model
+    (pair table), all with split contexts: their partials, counters and the
+    table live in one workspace and must not overlap.  Run twice to check that
+    the counters come back to zero."""
+    _announce("multi decode mixed G + large batch")
+    bs, N = 16, 30000
+    rng = np.random.Generator(np.random.PCG64(21))
+    shapes = [("gqa", 16, 2, rng.integers(1, 700, size=5)),
+              ("mha-small", 3, 3, rng.integers(1, 500, size=7)),
+              ("mha-large", 1, 1, rng.integers(1, 300, size=300))]
+    ids = rng.permutation(N)
+    models, cur = [], 0
+    for name, hq, hk, ctx in shapes:
+        bt, cur = workloads.build_tables(ctx.astype(np.int32), hk, bs, ids, cur)
+        models.append(workloads.DecodeModel(name, hq, hk, ctx.astype(np.int32), bt))
+    dk, dv = allocate_gpu_cache(N, bs, DEV)
+    dk.fill_(float("nan"))
+    dv.fill_(float("nan"))
+    workloads.fill_blocks(dk, dv, np.concatenate([m.used_blocks(bs) for m in models]), seed=21)
+    for i, m in enumerate(models):
+        m.to_device(DEV, torch.float16, seed=30 + i)
+    calls = [ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale)
+             for m in models]
+    ks, vs, tables = workloads.compact_to_host(dk, dv, models, bs)
+    for rep in range(2):
+        for m in models:
+            m.out.fill_(7.0)
+        ops.multi_decode(calls, dk, dv, partition_size=128)
+        torch.cuda.synchronize()
+        for m, t in zip(models, tables):
+            want = orc.paged_decode(m.q.cpu(), ks, vs, t, m.context_lens, m.scale)
+            _check(m.out[:m.batch].float().cpu(), want)
+
+
 def test_decode_rejects_bad_arguments():
     _announce("decode argument validation")
     dk, dv = allocate_gpu_cache(8, 16, DEV)
