@@ -251,21 +251,25 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
     for (int kb = 0; kb < 2; ++kb) {
       float p[16];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        p[i] = fast_exp2(__builtin_fmaf(sacc[kb][i], P.scale_log2, neg_m));
-        psum += p[i];
-      }
+      for (int i = 0; i < 16; ++i) p[i] = fast_exp2(__builtin_fmaf(sacc[kb][i], P.scale_log2, neg_m));
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
-        pf[2 * kb + st].u = u32x4{pack2<T>(p[8 * st + 0], p[8 * st + 1]), pack2<T>(p[8 * st + 2], p[8 * st + 3]),
-                                       pack2<T>(p[8 * st + 4], p[8 * st + 5]), pack2<T>(p[8 * st + 6], p[8 * st + 7])};
-        if constexpr (kSplitP) {
-          float r[8];
+        uint32_t w[4];
 #pragma unroll
-          for (int j = 0; j < 8; ++j)
-            r[j] = p[8 * st + j] - __uint_as_float(static_cast<uint32_t>(f32_to_bf16_bits(p[8 * st + j])) << 16);
-          pf_lo[2 * kb + st].u = u32x4{pack2<T>(r[0], r[1]), pack2<T>(r[2], r[3]),
-                                            pack2<T>(r[4], r[5]), pack2<T>(r[6], r[7])};
+        for (int j = 0; j < 4; ++j) w[j] = pack2<T>(p[8 * st + 2 * j], p[8 * st + 2 * j + 1]);
+        pf[2 * kb + st].u = u32x4{w[0], w[1], w[2], w[3]};
+        if constexpr (kSplitP) {
+          // The part of p that its bf16 rounding lost, as a second bf16.
+          uint32_t lo[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            lo[j] = pack2<T>(p[8 * st + 2 * j] - bf16_lo(w[j]), p[8 * st + 2 * j + 1] - bf16_hi(w[j]));
+            psum += p[8 * st + 2 * j] + p[8 * st + 2 * j + 1];
+          }
+          pf_lo[2 * kb + st].u = u32x4{lo[0], lo[1], lo[2], lo[3]};
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) psum += p[8 * st + j];
         }
       }
     }
