@@ -173,6 +173,21 @@ int32_t mux_rotary_neox(const int64_t *positions, void *q, int64_t q_row_stride,
                         int32_t rotary_dim, int32_t num_tokens, int32_t num_q_heads,
                         int32_t num_kv_heads, int32_t head_size, int32_t dtype, void *stream);
 
+/* The same rotation fused with the cache write (the two steps that open the
+ * attention layer's forward, models/llama.py:159-161): q and k of the first
+ * num_tokens rows are rotated in place and the rotated k, with v, is scattered
+ * through slot_mapping as by mux_reshape_and_cache - one launch and one pass
+ * over k.  Rows without a slot (< 0) are still rotated.  rotary_dim must be
+ * head_size (128), q/k/v 16-byte aligned with row strides that are multiples
+ * of 8; q may be NULL (k only). */
+int32_t mux_rope_reshape_and_cache(const int64_t *positions, void *q, int64_t q_row_stride, void *k,
+                                   const void *v, int64_t kv_row_stride, const float *cos_sin,
+                                   int32_t max_position, int32_t rotary_dim, void *k_pool, void *v_pool,
+                                   int64_t num_pool_blocks, const int64_t *slot_mapping, int32_t layer,
+                                   int32_t num_layers, int32_t num_tokens, int32_t num_q_heads,
+                                   int32_t num_kv_heads, int32_t head_size, int32_t block_size,
+                                   int32_t dtype, void *stream);
+
 /* ---- CU-masked streams ---------------------------------------------------
  * Replacement for the reference's per-process MPS share
  * (CUDA_MPS_ACTIVE_THREAD_PERCENTAGE, muxserve/muxsched/launcher.py:54-61):

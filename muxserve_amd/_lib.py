@@ -127,6 +127,8 @@ ATTN_SIGNATURES = {
                                    c_i32, c_i32, c_i32, c_f32, c_i32, c_vp]),
     "mux_rotary_neox": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32,
                                 c_i32, c_vp]),
+    "mux_rope_reshape_and_cache": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i32, c_i32, c_vp, c_vp, c_i64,
+                                           c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp]),
     "mux_stream_create_cu_range": (c_i32, [c_vp, c_i32, c_i32, c_vp]),
     "mux_stream_destroy": (c_i32, [c_vp]),
     "mux_device_cu_info": (c_i32, [c_vp]),

@@ -19,17 +19,60 @@
 // token 16w, if there is one: both neighbours derive it from the same slots,
 // the windows still tile the token stream exactly, each holds 9..23 tokens,
 // and no run straddles two workgroups.
+//
+// Fused variant (ROPE): the same kernel first applies the NeoX rotary embedding
+// to k (and to the query heads that share this kv head) for the tokens of its
+// window, in place, and scatters the rotated k - one launch and one pass over k
+// instead of a rotary kernel followed by the cache write.  A thread's chunk c
+// pairs with chunk c^8 (dims +-64) of the same token: both are read, the
+// workgroup meets, then the rotated chunk goes back in place and into the pool.
 #include "mux_common.h"
 
 namespace mux {
 
+struct RopeArgs {
+  uint16_t *q;                 // rotated in place; may be null
+  int64_t q_stride;
+  int32_t ratio;               // query heads per kv head
+  const int64_t *positions;    // [num_tokens]
+  const float *cos_sin;        // [max_position, 128] = [cos | sin]
+  int32_t max_position;
+};
+
+// out = own * cos + (is_y ? +1 : -1) * partner * sin, elementwise on 8 packed values.
+template <typename T>
+__device__ __forceinline__ uint4 rotate_chunk(const uint4 own, const uint4 partner, const float (&cs)[8],
+                                              const float (&sn)[8], bool is_y) {
+  const uint32_t a[4] = {own.x, own.y, own.z, own.w};
+  const uint32_t b[4] = {partner.x, partner.y, partner.z, partner.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float a0, a1, b0, b1;
+    if constexpr (__is_same(T, F16)) {
+      const half2_t ah = as_half2(a[e]), bh = as_half2(b[e]);
+      a0 = static_cast<float>(ah.x); a1 = static_cast<float>(ah.y);
+      b0 = static_cast<float>(bh.x); b1 = static_cast<float>(bh.y);
+    } else {
+      a0 = bf16_lo(a[e]); a1 = bf16_hi(a[e]);
+      b0 = bf16_lo(b[e]); b1 = bf16_hi(b[e]);
+    }
+    // x' = x c - y s for the low half of a head, y' = y c + x s for the high half.
+    const float r0 = is_y ? a0 * cs[2 * e] + b0 * sn[2 * e] : a0 * cs[2 * e] - b0 * sn[2 * e];
+    const float r1 = is_y ? a1 * cs[2 * e + 1] + b1 * sn[2 * e + 1] : a1 * cs[2 * e + 1] - b1 * sn[2 * e + 1];
+    o[e] = static_cast<uint32_t>(to_storage<T>(r0)) | (static_cast<uint32_t>(to_storage<T>(r1)) << 16);
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 constexpr int kVtRow = kHeadSize + 8;    // LDS row of one token: 256 B + 16 B so that rows shift banks
 constexpr int kSlotWin = 40;             // slots of tokens 16w-8 .. 16w+31 are examined
 
+template <typename T, bool ROPE>
 __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
-    const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, int64_t row_stride,
+    uint16_t *k, const uint16_t *__restrict__ v, int64_t row_stride,
     uint4 *__restrict__ k_pool, uint16_t *__restrict__ v_pool, int64_t num_blocks,
-    const int64_t *__restrict__ slots, int64_t slot_stride, int num_tokens, int block_size) {
+    const int64_t *__restrict__ slots, int64_t slot_stride, int num_tokens, int block_size, const RopeArgs R) {
   constexpr int D = kHeadSize;
   __shared__ __attribute__((aligned(16))) uint16_t vt[24][kVtRow];
   __shared__ int64_t s_slot[kSlotWin + 8];
@@ -44,10 +87,12 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
   // first and overlap the slot examination.
   const int t_nom = T0 + i;
   const int64_t src_nom = static_cast<int64_t>(t_nom) * row_stride + h * D + c * 8;
-  uint4 kx = make_uint4(0, 0, 0, 0), vx = make_uint4(0, 0, 0, 0);
+  uint4 kx = make_uint4(0, 0, 0, 0), vx = make_uint4(0, 0, 0, 0), kpart = make_uint4(0, 0, 0, 0);
+  const int pc = (c ^ 8) - c;              // the partner chunk of the rotation, in chunks from this one
   if (t_nom < num_tokens) {
     kx = *reinterpret_cast<const uint4 *>(k + src_nom);
     vx = *reinterpret_cast<const uint4 *>(v + src_nom);
+    if constexpr (ROPE) kpart = *reinterpret_cast<const uint4 *>(k + src_nom + pc * 8);
   }
 
   // Slots of tokens T0-8 .. T0+31; -1 for tokens outside the batch, skipped
@@ -81,20 +126,62 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
     const int j = pass == 0 ? 8 + i : i;
+    const bool mine = j >= ja && j < jb && (pass == 0 || i < 8);     // token T0-8+j is in this window
+    const int t = T0 - 8 + j;
+    const int64_t src = static_cast<int64_t>(t) * row_stride + h * D + c * 8;
     if (pass == 1) {
-      if (i >= 8) break;
+      if (ja == 8) break;                // uniform: no token taken over from the previous workgroup
+      if constexpr (!ROPE) {
+        if (i >= 8) break;
+      }
       kx = make_uint4(0, 0, 0, 0);
       vx = make_uint4(0, 0, 0, 0);
+      kpart = make_uint4(0, 0, 0, 0);
     }
-    const int64_t slot = (j >= ja && j < jb) ? s_slot[j] : -1;
+    const int64_t slot = mine ? s_slot[j] : -1;
+    if (pass == 1 && mine && (ROPE || slot >= 0)) {
+      kx = *reinterpret_cast<const uint4 *>(k + src);
+      vx = *reinterpret_cast<const uint4 *>(v + src);
+      if constexpr (ROPE) kpart = *reinterpret_cast<const uint4 *>(k + src + pc * 8);
+    }
+    if constexpr (ROPE) {
+      // Rotate k of every token of the window (also tokens without a slot), and
+      // the query heads of this kv head, four at a time; all reads of a group
+      // precede its writes (the workgroup meets in between), because a thread's
+      // partner chunk is another thread's own.
+      float cs[8], sn[8];
+      if (mine) {
+        int64_t pos = R.positions[t];
+        pos = pos < 0 ? 0 : (pos >= R.max_position ? R.max_position - 1 : pos);
+        const float *row = R.cos_sin + pos * D + (c & 7) * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          cs[e] = row[e];
+          sn[e] = row[D / 2 + e];
+        }
+        kx = rotate_chunk<T>(kx, kpart, cs, sn, c >= 8);
+      }
+      const int n_q = R.q != nullptr ? R.ratio : 0;
+      uint16_t *q0 = R.q + static_cast<int64_t>(t) * R.q_stride + static_cast<int64_t>(h) * R.ratio * D + c * 8;
+      for (int g0 = 0; g0 < max(n_q, 1); g0 += 4) {
+        uint4 qx[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          if (mine && g0 + g < n_q) {
+            const uint16_t *qp = q0 + (g0 + g) * D;
+            qx[g] = rotate_chunk<T>(*reinterpret_cast<const uint4 *>(qp),
+                                    *reinterpret_cast<const uint4 *>(qp + pc * 8), cs, sn, c >= 8);
+          }
+        __syncthreads();
+        if (mine && g0 == 0) *reinterpret_cast<uint4 *>(k + src) = kx;
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          if (mine && g0 + g < n_q) *reinterpret_cast<uint4 *>(q0 + (g0 + g) * D) = qx[g];
+      }
+    }
     if (slot >= 0) {
       const int64_t blk = slot / block_size;
       const int o = static_cast<int>(slot - blk * block_size);
-      if (pass == 1) {
-        const int64_t src = static_cast<int64_t>(T0 - 8 + j) * row_stride + h * D + c * 8;
-        kx = *reinterpret_cast<const uint4 *>(k + src);
-        vx = *reinterpret_cast<const uint4 *>(v + src);
-      }
       k_pool[(blk * (D / 8) + c) * block_size + o] = kx;
       // Element path for tokens that no run covers (a run starts at most 7 tokens back).
       const uint32_t cover = in_win & (0xffu << (j > 7 ? j - 7 : 0)) & ~(~0u << (j + 1));
@@ -108,7 +195,7 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
         }
       }
     }
-    if (in_win != 0) *reinterpret_cast<uint4 *>(&vt[j][c * 8]) = vx;
+    if (in_win != 0 && (pass == 0 || i < 8)) *reinterpret_cast<uint4 *>(&vt[j][c * 8]) = vx;
   }
   if (in_win == 0) return;                                 // uniform: no run in this window
   __syncthreads();
@@ -131,12 +218,13 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
 
 }  // namespace mux
 
-extern "C" int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t kv_row_stride,
-                                         void *k_pool, void *v_pool, int64_t num_pool_blocks,
-                                         const int64_t *slot_mapping, int32_t layer, int32_t num_layers,
-                                         int32_t num_tokens, int32_t num_kv_heads, int32_t head_size,
-                                         int32_t block_size, int32_t dtype, void *stream) {
-  using namespace mux;
+namespace mux {
+namespace {
+
+int32_t check_cache_write(const void *k, const void *v, int64_t kv_row_stride, const void *k_pool,
+                          const void *v_pool, int64_t num_pool_blocks, const int64_t *slot_mapping, int32_t layer,
+                          int32_t num_layers, int32_t num_tokens, int32_t num_kv_heads, int32_t head_size,
+                          int32_t block_size, int32_t dtype) {
   if (!k || !v || !k_pool || !v_pool || !slot_mapping) return MUXA_EINVAL;
   if (num_tokens < 0 || num_kv_heads <= 0 || num_pool_blocks <= 0) return MUXA_EINVAL;
   if (layer < 0 || layer >= num_layers) return MUXA_EINVAL;
@@ -150,14 +238,73 @@ extern "C" int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t k
   if (align & 15u) return MUXA_EINVAL;
   if (num_kv_heads > 65535) return MUXA_EUNSUPPORTED;
   if (num_pool_blocks > (int64_t{1} << 56)) return MUXA_EINVAL;   // slot arithmetic stays in 64 bits
+  return MUXA_OK;
+}
+
+}  // namespace
+}  // namespace mux
+
+extern "C" int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t kv_row_stride,
+                                         void *k_pool, void *v_pool, int64_t num_pool_blocks,
+                                         const int64_t *slot_mapping, int32_t layer, int32_t num_layers,
+                                         int32_t num_tokens, int32_t num_kv_heads, int32_t head_size,
+                                         int32_t block_size, int32_t dtype, void *stream) {
+  using namespace mux;
+  const int32_t rc = check_cache_write(k, v, kv_row_stride, k_pool, v_pool, num_pool_blocks, slot_mapping, layer,
+                                       num_layers, num_tokens, num_kv_heads, head_size, block_size, dtype);
+  if (rc != MUXA_OK) return rc;
   if (num_tokens == 0) return MUXA_OK;
   const int64_t slot_stride = static_cast<int64_t>(num_layers) * num_kv_heads;
   const int64_t *slots = slot_mapping + static_cast<int64_t>(layer) * num_kv_heads;
   dim3 grid((num_tokens + 15) / 16, num_kv_heads);
-  hipLaunchKernelGGL(reshape_and_cache_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const uint16_t *>(k), static_cast<const uint16_t *>(v), kv_row_stride,
-                     static_cast<uint4 *>(k_pool), static_cast<uint16_t *>(v_pool), num_pool_blocks,
-                     slots, slot_stride, num_tokens, block_size);
+  // Without the rotary part the kernel only moves bytes and never writes k.
+  hipLaunchKernelGGL((reshape_and_cache_kernel<F16, false>), grid, dim3(256), 0, static_cast<hipStream_t>(stream),
+                     const_cast<uint16_t *>(static_cast<const uint16_t *>(k)), static_cast<const uint16_t *>(v),
+                     kv_row_stride, static_cast<uint4 *>(k_pool), static_cast<uint16_t *>(v_pool), num_pool_blocks,
+                     slots, slot_stride, num_tokens, block_size, RopeArgs{});
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(e);
+  return MUXA_OK;
+}
+
+extern "C" int32_t mux_rope_reshape_and_cache(const int64_t *positions, void *q, int64_t q_row_stride, void *k,
+                                              const void *v, int64_t kv_row_stride, const float *cos_sin,
+                                              int32_t max_position, int32_t rotary_dim, void *k_pool, void *v_pool,
+                                              int64_t num_pool_blocks, const int64_t *slot_mapping, int32_t layer,
+                                              int32_t num_layers, int32_t num_tokens, int32_t num_q_heads,
+                                              int32_t num_kv_heads, int32_t head_size, int32_t block_size,
+                                              int32_t dtype, void *stream) {
+  using namespace mux;
+  const int32_t rc = check_cache_write(k, v, kv_row_stride, k_pool, v_pool, num_pool_blocks, slot_mapping, layer,
+                                       num_layers, num_tokens, num_kv_heads, head_size, block_size, dtype);
+  if (rc != MUXA_OK) return rc;
+  if (!positions || !cos_sin || max_position <= 0) return MUXA_EINVAL;
+  if (rotary_dim != kHeadSize) return MUXA_EUNSUPPORTED;   // partial rotation: use mux_rotary_neox + mux_reshape_and_cache
+  if (q != nullptr) {
+    if (num_q_heads <= 0 || num_q_heads % num_kv_heads != 0) return MUXA_EINVAL;
+    if (q_row_stride < static_cast<int64_t>(num_q_heads) * kHeadSize || q_row_stride % 8 != 0) return MUXA_EINVAL;
+    if (reinterpret_cast<uintptr_t>(q) & 15u) return MUXA_EINVAL;
+  }
+  if (num_tokens == 0) return MUXA_OK;
+  const int64_t slot_stride = static_cast<int64_t>(num_layers) * num_kv_heads;
+  const int64_t *slots = slot_mapping + static_cast<int64_t>(layer) * num_kv_heads;
+  RopeArgs R;
+  R.q = static_cast<uint16_t *>(q);
+  R.q_stride = q_row_stride;
+  R.ratio = q ? num_q_heads / num_kv_heads : 0;
+  R.positions = positions;
+  R.cos_sin = cos_sin;
+  R.max_position = max_position;
+  dim3 grid((num_tokens + 15) / 16, num_kv_heads);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == MUXA_DTYPE_F16)
+    hipLaunchKernelGGL((reshape_and_cache_kernel<F16, true>), grid, dim3(256), 0, st, static_cast<uint16_t *>(k),
+                       static_cast<const uint16_t *>(v), kv_row_stride, static_cast<uint4 *>(k_pool),
+                       static_cast<uint16_t *>(v_pool), num_pool_blocks, slots, slot_stride, num_tokens, block_size, R);
+  else
+    hipLaunchKernelGGL((reshape_and_cache_kernel<BF16, true>), grid, dim3(256), 0, st, static_cast<uint16_t *>(k),
+                       static_cast<const uint16_t *>(v), kv_row_stride, static_cast<uint4 *>(k_pool),
+                       static_cast<uint16_t *>(v_pool), num_pool_blocks, slots, slot_stride, num_tokens, block_size, R);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e);
   return MUXA_OK;

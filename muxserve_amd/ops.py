@@ -211,6 +211,41 @@ def rotary_neox(positions: torch.Tensor, q: torch.Tensor, k: torch.Tensor, cos_s
     _lib.check_attn(rc, "mux_rotary_neox")
 
 
+def rope_reshape_and_cache(positions: torch.Tensor, q: Optional[torch.Tensor], k: torch.Tensor, v: torch.Tensor,
+                           cos_sin: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                           slot_mapping: torch.Tensor, layer: int = 0, num_tokens: Optional[int] = None,
+                           stream=None) -> None:
+    """rotary_neox (rotary_dim = 128) on q and k in place, then reshape_and_cache
+    of the rotated k and v, in one launch.  Same results as the two calls."""
+    _need_cuda(positions, k, v, cos_sin, k_pool, v_pool, slot_mapping)
+    bs = _check_pools(k_pool, v_pool)
+    if positions.dtype != torch.int64 or positions.dim() != 1 or not positions.is_contiguous():
+        raise ValueError("positions: expected contiguous int64 [T]")
+    if cos_sin.dtype != torch.float32 or cos_sin.dim() != 2 or not cos_sin.is_contiguous():
+        raise ValueError("cos_sin: expected contiguous float32 [max_position, rotary_dim]")
+    if slot_mapping.dtype != torch.int64 or slot_mapping.dim() != 3 or not slot_mapping.is_contiguous():
+        raise ValueError("slot_mapping: expected contiguous int64 [T, L, Hkv]")
+    T, L, H = slot_mapping.shape
+    if num_tokens is not None:
+        T = min(T, int(num_tokens))
+    stride = _rows(k, "k")
+    if _rows(v, "v") != stride or k.shape != v.shape or k.dtype != v.dtype or k.dtype != k_pool.dtype:
+        raise ValueError("k and v must have the same shape, strides and dtype as each other and the pool's dtype")
+    if k.shape[0] < T or positions.shape[0] < T or k.shape[1] != H * HEAD_SIZE:
+        raise ValueError(f"k: expected [>={T}, {H * HEAD_SIZE}], got {tuple(k.shape)}")
+    q_ptr, q_stride, hq = None, 0, 0
+    if q is not None:
+        _need_cuda(q)
+        if q.dtype != k.dtype or q.shape[1] % HEAD_SIZE or q.shape[0] < T:
+            raise ValueError("q [>=T, Hq*128] of the dtype of k expected")
+        q_ptr, q_stride, hq = q.data_ptr(), _rows(q, "q"), q.shape[1] // HEAD_SIZE
+    rc = _lib.attn().mux_rope_reshape_and_cache(
+        positions.data_ptr(), q_ptr, q_stride, k.data_ptr(), v.data_ptr(), stride, cos_sin.data_ptr(),
+        cos_sin.shape[0], cos_sin.shape[1], k_pool.data_ptr(), v_pool.data_ptr(), k_pool.shape[0],
+        slot_mapping.data_ptr(), int(layer), L, T, hq, H, HEAD_SIZE, bs, _dtype_code(k), _stream_ptr(stream))
+    _lib.check_attn(rc, "mux_rope_reshape_and_cache")
+
+
 class CUMaskedStream:
     """A HIP stream restricted to a share of the GPU's compute units (the
     replacement for a per-process MPS percentage).  Usable wherever a stream is

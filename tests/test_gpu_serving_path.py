@@ -10,6 +10,7 @@ import pytest
 import torch
 
 from oracle import attn_oracle as orc
+from muxserve_amd import ops
 from muxserve_amd.attention import PagedAttentionWithRoPE
 from muxserve_amd.batch_scheduler import BatchScheduler
 from muxserve_amd.memory_manager import KVStorage
@@ -23,12 +24,14 @@ TOL = 2e-3
 
 
 class _Model:
-    def __init__(self, name, L, Hq, Hkv, storage, bs, seed):
+    def __init__(self, name, L, Hq, Hkv, storage, bs, seed, fused_rope_max_tokens=512):
         self.name, self.L, self.Hq, self.Hkv = name, L, Hq, Hkv
         self.sched = BatchScheduler(L, Hkv, 512, bs)
         self.storage = storage
         self.layers = [PagedAttentionWithRoPE(Hq, D, D ** -0.5, base=10000, max_position=2048, rotary_dim=D,
                                               num_kv_heads=Hkv, rope_scaling=None, layer_idx=l) for l in range(L)]
+        for layer in self.layers:
+            layer.fused_rope_max_tokens = fused_rope_max_tokens
         self.g = torch.Generator().manual_seed(seed)
 
     def alloc(self, req):
@@ -69,17 +72,19 @@ def _step(m, ids, last_tokens, k_pool, v_pool, hk, hv, permuted):
     return worst
 
 
-@pytest.mark.parametrize("permuted", [True, False])
-def test_two_models_share_one_pool_prefill_then_decode(permuted):
-    print(f"[case] serving path permuted_tables={permuted}", flush=True)
+@pytest.mark.parametrize("permuted,fused_max", [(True, 512), (False, 512), (True, 0), (True, 60)])
+def test_two_models_share_one_pool_prefill_then_decode(permuted, fused_max):
+    """fused_max: steps of up to that many tokens rotate and write the cache in
+    one launch (0: always the two kernels; 60: decode steps fused, prefill not)."""
+    print(f"[case] serving path permuted_tables={permuted} fused_rope_max_tokens={fused_max}", flush=True)
     bs, N = 16, 6000
     storage = KVStorage(N)
     k_pool, v_pool = allocate_gpu_cache(N, bs, DEV)
     k_pool.zero_()
     v_pool.zero_()
     hk, hv = k_pool.cpu(), v_pool.cpu()
-    a = _Model("small-mha", 2, 4, 4, storage, bs, seed=1)
-    b = _Model("gqa", 3, 8, 2, storage, bs, seed=2)
+    a = _Model("small-mha", 2, 4, 4, storage, bs, seed=1, fused_rope_max_tokens=fused_max)
+    b = _Model("gqa", 3, 8, 2, storage, bs, seed=2, fused_rope_max_tokens=fused_max)
     rng = np.random.Generator(np.random.PCG64(3))
     for m, lens, base_id in ((a, [5, 40, 17], 0), (b, [130, 16, 1, 33], 100)):
         for i, p in enumerate(lens):
@@ -101,3 +106,47 @@ def test_two_models_share_one_pool_prefill_then_decode(permuted):
     assert torch.equal(k_pool.cpu().view(torch.int16), hk.view(torch.int16))
     assert torch.equal(v_pool.cpu().view(torch.int16), hv.view(torch.int16))
     assert storage.num_free() + sum(storage.num_held(i) for i in [0, 2, 100, 101, 102, 103, 104]) == N
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv", [(3, 3), (8, 2)])
+@pytest.mark.parametrize("bs", [16, 8])
+def test_fused_rotary_cache_write_equals_the_two_kernels(dtype, Hq, Hkv, bs):
+    """mux_rope_reshape_and_cache against mux_rotary_neox followed by
+    mux_reshape_and_cache on the same inputs: q, k and both pools bitwise equal.
+    Packed ragged prompts (runs at every phase) plus tokens without a slot,
+    which are rotated but not written."""
+    print(f"[case] fused rope + cache write {dtype} Hq={Hq} Hkv={Hkv} bs={bs}", flush=True)
+    from muxserve_amd import workloads
+    from muxserve_amd.attention import build_cos_sin_cache
+    from muxserve_amd.pool import allocate_gpu_cache
+    rng = np.random.Generator(np.random.PCG64(77 + bs))
+    g = torch.Generator().manual_seed(77 + bs)
+    lens = rng.permutation(np.arange(1, 30)).astype(np.int32)
+    T = int(lens.sum())
+    N = int(((lens + bs - 1) // bs).sum()) * Hkv + 5
+    slots, _ = workloads.prefill_slot_mapping(lens, Hkv, bs, rng.permutation(N))
+    slots[5, 0, 0] = -1
+    slots[T - 1, 0, :] = -1
+    pad = (T + 7) // 8 * 8
+    qkv = torch.randn((pad, (Hq + 2 * Hkv) * D), generator=g).to(dtype).to(DEV)
+    positions = torch.from_numpy(rng.integers(0, 2048, size=pad)).to(DEV)
+    cos_sin = build_cos_sin_cache(D, 2048, 10000.0, DEV)
+    dslots = torch.from_numpy(slots).to(DEV)
+    results = []
+    for fused in (False, True):
+        x = qkv.clone()
+        q, k, v = x.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+        kp, vp = allocate_gpu_cache(N, bs, DEV, dtype=dtype)
+        kp.zero_()
+        vp.zero_()
+        if fused:
+            ops.rope_reshape_and_cache(positions, q, k, v, cos_sin, kp, vp, dslots, num_tokens=T)
+        else:
+            ops.rotary_neox(positions, q, k, cos_sin, num_tokens=T)
+            ops.reshape_and_cache(k, v, kp, vp, dslots, num_tokens=T)
+        torch.cuda.synchronize()
+        results.append((x.cpu().view(torch.int16), kp.cpu().view(torch.int16), vp.cpu().view(torch.int16)))
+    for a, b, what in zip(results[0], results[1], ("qkv rows", "k pool", "v pool")):
+        assert torch.equal(a, b), f"{what} differ between the fused launch and the two kernels"
+    assert torch.equal(results[1][0][T:], qkv.cpu().view(torch.int16)[T:]), "padding rows must not be touched"
