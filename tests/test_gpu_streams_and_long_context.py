@@ -82,3 +82,86 @@ def test_long_context_gqa_bf16_full_size_pool():
     got = m.out[pick].float().cpu()
     bound = 2e-3 + want.abs() * 2.0 ** -8          # + rounding of the bf16 result
     assert ((got - want).abs() - bound).max().item() <= 0, (got - want).abs().max().item()
+
+
+def test_decode_step_replays_from_a_hip_graph():
+    """Cache write (fused with rotary) + fused three-model decode with split
+    contexts and a 300-sequence model, captured once and replayed with new
+    inputs; eager work and synchronisations between replays; every replay must
+    equal the eager result bitwise (the split workspace's counters have to be
+    back at zero after every run, eager or replayed)."""
+    print("[case] hip graph replay of a decode step", flush=True)
+    from muxserve_amd import _lib
+    from muxserve_amd.attention import build_cos_sin_cache
+    import ctypes
+    bs, N = 16, 60000
+    rng = np.random.Generator(np.random.PCG64(31))
+    k_pool, v_pool = allocate_gpu_cache(N, bs, DEV)
+    k_pool.zero_()
+    v_pool.zero_()
+    shapes = [("a", 4, 4, rng.integers(1, 900, size=6)), ("gqa", 8, 1, rng.integers(1, 900, size=5)),
+              ("big", 1, 1, rng.integers(1, 400, size=300))]
+    ids = rng.permutation(N)
+    models, cur = [], 0
+    for name, hq, hk, ctx in shapes:
+        bt, cur = workloads.build_tables(ctx.astype(np.int32), hk, bs, ids, cur)
+        models.append(workloads.DecodeModel(name, hq, hk, ctx.astype(np.int32), bt).to_device(DEV, torch.float16, seed=cur))
+    workloads.fill_blocks(k_pool, v_pool, np.concatenate([m.used_blocks(bs) for m in models]), seed=31)
+    calls = [ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale)
+             for m in models]
+    items = (_lib.MuxDecodeItem * len(calls))(*[c.to_item() for c in calls])
+    need = _lib.attn().mux_paged_decode_workspace_bytes(ctypes.addressof(items), len(calls), 128)
+    ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    # the new token of model "a": k, v rows and the slot of its last context position
+    a = models[0]
+    cos_sin = build_cos_sin_cache(D, 2048, 10000.0, DEV)
+    kv = torch.zeros((8, 2 * a.num_kv_heads * D), dtype=torch.float16, device=DEV)
+    positions = torch.from_numpy(np.pad(a.context_lens.astype(np.int64) - 1, (0, 8 - a.batch))).to(DEV)
+    last = (a.context_lens - 1)
+    slots = (a.block_tables[0, np.arange(a.batch), :, last // bs].astype(np.int64) * bs + (last % bs)[:, None])
+    dslots = torch.from_numpy(slots[:, None, :].copy()).to(DEV)
+
+    def step():
+        ops.rope_reshape_and_cache(positions, a.q, kv[:, :a.num_kv_heads * D], kv[:, a.num_kv_heads * D:], cos_sin,
+                                   k_pool, v_pool, dslots, num_tokens=a.batch)
+        ops.multi_decode(calls, k_pool, v_pool, partition_size=128, workspace=ws)
+
+    def new_inputs(seed):
+        g = torch.Generator(device=DEV).manual_seed(seed)
+        for m in models:
+            m.q.copy_(torch.randn(m.q.shape, generator=g, device=DEV).half())
+        kv.copy_(torch.randn(kv.shape, generator=g, device=DEV).half())
+
+    stream = torch.cuda.Stream()
+    new_inputs(0)
+    with torch.cuda.stream(stream):
+        step()                                  # warm-up outside capture
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    new_inputs(1)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=stream):
+        step()
+    for rep in range(4):
+        new_inputs(10 + rep)
+        q_before = [m.q.clone() for m in models]
+        kv_before = kv.clone()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [m.out.clone() for m in models]
+        pools = (k_pool.clone(), v_pool.clone())
+        # eager run on the same inputs (q and k of model a were rotated in place by the replay: restore them)
+        kv.copy_(kv_before)
+        for m, q0 in zip(models, q_before):
+            m.q.copy_(q0)
+            m.out.zero_()
+        step()
+        torch.cuda.synchronize()
+        for m, o in zip(models, got):
+            assert torch.equal(o, m.out), f"replay {rep}: model {m.name} differs from the eager run"
+        assert torch.equal(pools[0], k_pool) and torch.equal(pools[1], v_pool)
+    ks, vs, tables = workloads.compact_to_host(k_pool, v_pool, models, bs)
+    for m, t in zip(models, tables):
+        want = orc.paged_decode(m.q.cpu(), ks, vs, t, m.context_lens, m.scale)
+        assert (m.out[:m.batch].float().cpu() - want).abs().max().item() <= 2e-3
