@@ -90,6 +90,14 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// K/V blocks are read exactly once per launch: non-temporal loads keep them
+// from displacing the block tables, q and context lengths in the XCD's L2.
+typedef uint32_t nt_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 stream_load(const uint4 *p) {
+  const nt_u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const nt_u32x4 *>(p));
+  return make_uint4(t.x, t.y, t.z, t.w);
+}
+
 template <int BS>
 struct Geometry {
   static_assert(BS == 8 || BS == 16 || BS == 32, "block size");
@@ -122,7 +130,7 @@ __device__ __forceinline__ void issue_tile_loads(uint4 (&kreg)[16], uint4 (&vreg
   if (tok < t1) {
     const uint4 *kp = kpool + static_cast<int64_t>(id) * Geo::BLOCK_CHUNKS + (tok % BS);
 #pragma unroll
-    for (int j = 0; j < 16; ++j) kreg[j] = kp[j * BS];
+    for (int j = 0; j < 16; ++j) kreg[j] = stream_load(&kp[j * BS]);
   } else {
 #pragma unroll
     for (int j = 0; j < 16; ++j) kreg[j] = make_uint4(0, 0, 0, 0);
@@ -134,7 +142,7 @@ __device__ __forceinline__ void issue_tile_loads(uint4 (&kreg)[16], uint4 (&vreg
     const bool chunk_ok = tb + b * BS + part * 8 < t1;
 #pragma unroll
     for (int j = 0; j < Geo::VI; ++j) {
-      if (chunk_ok) vreg[b][j] = vp[j * 64];
+      if (chunk_ok) vreg[b][j] = stream_load(&vp[j * 64]);
       else vreg[b][j] = make_uint4(0, 0, 0, 0);
     }
   }
@@ -795,12 +803,14 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
       const int tok = tb + 16 * tg + h;
       const u32x4_t *kp = kpool + static_cast<int64_t>(tg ? id.y : id.x) * Geo::BLOCK_CHUNKS + (tok % BS);
 #pragma unroll
-      for (int s = 0; s < 4; ++s) r.k[tg][s] = tok < t1 ? kp[(4 * s + g) * BS] : u32x4_t{0, 0, 0, 0};
+      for (int s = 0; s < 4; ++s)
+        r.k[tg][s] = tok < t1 ? __builtin_nontemporal_load(&kp[(4 * s + g) * BS]) : u32x4_t{0, 0, 0, 0};
     }
     const int tok = tb + 8 * g;
     const u32x4_t *vp = vpool + static_cast<int64_t>(id.z) * Geo::BLOCK_CHUNKS + (tok % BS) / 8;
 #pragma unroll
-    for (int nb = 0; nb < 8; ++nb) r.v[nb] = tok < t1 ? vp[(16 * nb + h) * Geo::PARTS] : u32x4_t{0, 0, 0, 0};
+    for (int nb = 0; nb < 8; ++nb)
+      r.v[nb] = tok < t1 ? __builtin_nontemporal_load(&vp[(16 * nb + h) * Geo::PARTS]) : u32x4_t{0, 0, 0, 0};
   };
   auto compute = [&](GqaTile &r, int tb) {
     const bool tail = tb + kGqaTile > t1;
