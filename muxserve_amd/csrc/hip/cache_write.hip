@@ -65,6 +65,23 @@ __device__ __forceinline__ uint4 rotate_chunk(const uint4 own, const uint4 partn
   return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
+// Stores that fill whole 128-byte lines by themselves go out non-temporal
+// (nothing to merge with, and the pool is not read back soon): K rows of a run
+// of 8 consecutive slots, V rows when the workgroup holds every run of the row.
+typedef uint32_t cw_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store16(void *p, const uint4 x, bool streaming) {
+  const cw_u32x4 v = {x.x, x.y, x.z, x.w};
+  if (streaming) {
+    // Written as an instruction: as two C++ stores that differ only in the hint,
+    // the optimiser folds the branches into one store and drops it.  The s_nop
+    // covers the wait state between a 16-byte store and a write of its data
+    // registers.
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 0" ::"v"(p), "v"(v) : "memory");
+  } else {
+    *static_cast<cw_u32x4 *>(p) = v;
+  }
+}
+
 constexpr int kVtRow = kHeadSize + 8;    // LDS row of one token: 256 B + 16 B so that rows shift banks
 constexpr int kSlotWin = 40;             // slots of tokens 16w-8 .. 16w+31 are examined
 
@@ -120,6 +137,16 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
   const int ja = before_lo ? __ffs(before_lo) - 1 : 8;
   const int jb = before_hi ? __ffs(before_hi) - 1 : min(24, num_tokens - T0 + 8);
   const uint32_t in_win = starts & (~0u << ja) & ~(~0u << jb);   // runs that start inside the window
+  // Does this window write whole pool rows and nothing else?  K rows of a run are
+  // 128 bytes; a V row is block_size * 2 bytes: one run fills it at block size 8,
+  // the two runs of a block at 16, never at 32.  Such a window streams its stores
+  // past the L2 (uniform over the workgroup).
+  const uint32_t second = in_win & (in_win - 1);
+  const int n_runs = __popc(in_win);
+  const bool rows_complete =
+      n_runs > 0 && jb - ja == 8 * n_runs &&
+      (block_size == 8 || (block_size == 16 && n_runs == 2 && __ffs(second) - __ffs(in_win) == 8 &&
+                           (s_slot[__ffs(in_win) - 1] & 15) == 0));
 
   // Rows of the LDS tile are bit positions: 8 + i for the nominal tokens, i for
   // the up to 7 tokens taken over from the previous workgroup's nominal range.
@@ -182,9 +209,9 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
     if (slot >= 0) {
       const int64_t blk = slot / block_size;
       const int o = static_cast<int>(slot - blk * block_size);
-      k_pool[(blk * (D / 8) + c) * block_size + o] = kx;
       // Element path for tokens that no run covers (a run starts at most 7 tokens back).
       const uint32_t cover = in_win & (0xffu << (j > 7 ? j - 7 : 0)) & ~(~0u << (j + 1));
+      store16(&k_pool[(blk * (D / 8) + c) * block_size + o], kx, rows_complete);
       if (cover == 0) {
         uint16_t *vp = v_pool + (blk * D + c * 8) * block_size + o;
         const uint32_t w[4] = {vx.x, vx.y, vx.z, vx.w};
@@ -212,7 +239,7 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
     const int64_t slot0 = s_slot[jp];
     const int64_t b0 = slot0 / block_size;
     const int o0 = static_cast<int>(slot0 - b0 * block_size);
-    *reinterpret_cast<uint4 *>(v_pool + (b0 * D + d) * block_size + o0) = make_uint4(w[0], w[1], w[2], w[3]);
+    store16(v_pool + (b0 * D + d) * block_size + o0, make_uint4(w[0], w[1], w[2], w[3]), rows_complete);
   }
 }
 
