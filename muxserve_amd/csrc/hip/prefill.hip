@@ -73,13 +73,16 @@ struct PrefillParams {
   int32_t num_kv_heads;
   int32_t num_groups;     // (prompt, kv head) pairs
   float scale_log2;
+  int32_t out_rows_16b;   // out and its row stride allow 16-byte stores
 };
 
 template <typename T>
 __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillParams P) {
   constexpr int D = kHeadSize;
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[kBN * kKRow];
-  __shared__ __attribute__((aligned(16))) uint16_t Vt[D * kVRow];
+  // One buffer: the K tile, then the V^T tile; the epilogue reuses all of it.
+  __shared__ __attribute__((aligned(16))) uint16_t smem[kBN * kKRow + D * kVRow];
+  uint16_t *const Ks = smem;
+  uint16_t *const Vt = smem + kBN * kKRow;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -314,8 +317,36 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
 
   // ---- normalise and store: register i of block mb is d = 32 mb + 8 (i/4) + 4 half + i%4 ------
   const float l_tot = l_run + __shfl_xor(l_run, 32);
-  if (my_q < len) {
-    const float inv = 1.f / l_tot;
+  const float inv = 1.f / l_tot;
+  if (P.out_rows_16b) {
+    // Through LDS, so that the rows go out as whole 256-byte runs (16 bytes per
+    // lane, four rows per instruction) instead of 8-byte pieces of 32 rows: the
+    // tile buffers are free once every wave has left the loop.
+    constexpr int kORow = D + 8;         // 272-byte rows
+    static_assert(4 * 32 * kORow <= kBN * kKRow + D * kVRow, "output staging fits the tile buffers");
+    __syncthreads();
+    uint16_t *stage = smem + wave * 32 * kORow;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        *reinterpret_cast<u32x2 *>(&stage[qcol * kORow + 32 * mb + 8 * g + 4 * half]) =
+            u32x2{pack2<T>(oacc[mb][4 * g] * inv, oacc[mb][4 * g + 1] * inv),
+                  pack2<T>(oacc[mb][4 * g + 2] * inv, oacc[mb][4 * g + 3] * inv)};
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int chunk = lane & 15;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int r = 4 * it + (lane >> 4);
+      if (wq0 + r < len) {
+        const u32x4 x = *reinterpret_cast<const u32x4 *>(&stage[r * kORow + 8 * chunk]);
+        *reinterpret_cast<u32x4 *>(P.out + static_cast<int64_t>(seq_begin + wq0 + r) * P.out_stride + hq * D +
+                                   8 * chunk) = x;
+      }
+    }
+  } else if (my_q < len) {
     uint16_t *op = P.out + static_cast<int64_t>(seq_begin + my_q) * P.out_stride + hq * D + 4 * half;
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb)
@@ -367,6 +398,7 @@ extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const v
   P.num_kv_heads = num_kv_heads;
   P.num_groups = num_prompts * num_kv_heads;
   P.scale_log2 = scale * 1.4426950408889634f;
+  P.out_rows_16b = (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && out_row_stride % 8 == 0;
   const int64_t n_wg = static_cast<int64_t>((P.num_groups + 7) / 8) * 8 * P.ratio * P.q_tiles;
   if (n_wg > 0x7fffffff) return MUXA_EUNSUPPORTED;
   const dim3 grid(static_cast<uint32_t>(n_wg));
