@@ -305,23 +305,26 @@ __device__ __forceinline__ void combine_head(const DecodeItemDev &I, int seq, in
 template <typename T, int G, int NW>
 __device__ __forceinline__ void merge_and_write(const DecodeItemDev &I, const Unit &u, int partition,
                                                 const float (*xa)[G][kHeadSize], const float (*xm)[G][2],
-                                                int lane) {
+                                                int n_active, int lane) {
   constexpr int D = kHeadSize;
   const bool single = u.ctx <= partition;
   const int hq0 = u.wh * G;
 #pragma unroll 1
   for (int g = 0; g < G; ++g) {
+    // Waves without tokens have left early and wrote nothing.
     float M = xm[0][g][0];
 #pragma unroll
-    for (int k = 1; k < NW; ++k) M = fmaxf(M, xm[k][g][0]);
+    for (int k = 1; k < NW; ++k)
+      if (k < n_active) M = fmaxf(M, xm[k][g][0]);
     float L = 0.f, a0 = 0.f, a1 = 0.f;
 #pragma unroll
-    for (int k = 0; k < NW; ++k) {
-      const float wgt = fast_exp2(xm[k][g][0] - M);
-      L += xm[k][g][1] * wgt;
-      a0 += xa[k][g][lane] * wgt;
-      a1 += xa[k][g][64 + lane] * wgt;
-    }
+    for (int k = 0; k < NW; ++k)
+      if (k < n_active) {
+        const float wgt = fast_exp2(xm[k][g][0] - M);
+        L += xm[k][g][1] * wgt;
+        a0 += xa[k][g][lane] * wgt;
+        a1 += xa[k][g][64 + lane] * wgt;
+      }
     const int hq = hq0 + g;
     if (single) {
       uint16_t *o = static_cast<uint16_t *>(I.out) + static_cast<int64_t>(u.seq) * I.out_stride + hq * D;
@@ -358,28 +361,31 @@ __device__ __forceinline__ void merge_and_write(const DecodeItemDev &I, const Un
 }
 
 // The same merge, publish and combine for a group of G heads, spread over the
-// workgroup's NW waves (wave w takes heads w, w+NW, ...).  Every wave of the
-// workgroup must call it.
+// workgroup's waves that had tokens (the first n_active; wave w takes heads w,
+// w + n_active, ...).  Every one of them must call it.
 template <typename T, int G, int NW>
 __device__ __forceinline__ void merge_and_write_group(const DecodeItemDev &I, const Unit &u, int partition,
                                                       const float (*xa)[G][kHeadSize], const float (*xm)[G][2],
-                                                      int *arrival_lds, int lane, int wave) {
+                                                      int *arrival_lds, int n_active, int lane, int wave) {
   constexpr int D = kHeadSize;
   const bool single = u.ctx <= partition;
   const int hq0 = u.wh * G;
 #pragma unroll 1
-  for (int g = wave; g < G; g += NW) {
+  for (int g = wave; g < G; g += n_active) {
+    // Waves without tokens have left early and wrote nothing.
     float M = xm[0][g][0];
 #pragma unroll
-    for (int k = 1; k < NW; ++k) M = fmaxf(M, xm[k][g][0]);
+    for (int k = 1; k < NW; ++k)
+      if (k < n_active) M = fmaxf(M, xm[k][g][0]);
     float L = 0.f, a0 = 0.f, a1 = 0.f;
 #pragma unroll
-    for (int k = 0; k < NW; ++k) {
-      const float wgt = fast_exp2(xm[k][g][0] - M);
-      L += xm[k][g][1] * wgt;
-      a0 += xa[k][g][lane] * wgt;
-      a1 += xa[k][g][64 + lane] * wgt;
-    }
+    for (int k = 0; k < NW; ++k)
+      if (k < n_active) {
+        const float wgt = fast_exp2(xm[k][g][0] - M);
+        L += xm[k][g][1] * wgt;
+        a0 += xa[k][g][lane] * wgt;
+        a1 += xa[k][g][64 + lane] * wgt;
+      }
     const int hq = hq0 + g;
     if (single) {
       uint16_t *o = static_cast<uint16_t *>(I.out) + static_cast<int64_t>(u.seq) * I.out_stride + hq * D;
@@ -410,7 +416,7 @@ __device__ __forceinline__ void merge_and_write_group(const DecodeItemDev &I, co
   if (*arrival_lds != n_splits - 1) return;
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 #pragma unroll 1
-  for (int g = wave; g < G; g += NW) combine_head<T>(I, u.seq, hq0 + g, n_splits, lane);
+  for (int g = wave; g < G; g += n_active) combine_head<T>(I, u.seq, hq0 + g, n_splits, lane);
   // Ready for the next launch.
   if (wave == 0 && lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -635,6 +641,10 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_kernel(const DecodeParam
   const uint4 *kpool = static_cast<const uint4 *>(P.k_pool);
   const uint4 *vpool = static_cast<const uint4 *>(P.v_pool);
   const int tb0 = u.t0 + wave * 64;
+  // A wave without tokens leaves at once and frees its registers for the next
+  // workgroup; the barrier below counts only the waves that are still there.
+  if (tb0 >= u.t1) return;
+  const int n_active = min(NW, (u.t1 - u.t0 + 63) / 64);
   int id_next = load_block_id<BS>(trow, tb0, u.t1, lane, P.last_block);
   uint32_t q_s[64];
   fetch_q<G>(I, u.seq, hq0, lane, q_s, q_lds[wave]);
@@ -658,7 +668,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_kernel(const DecodeParam
   stash_wave_partial<BS, G>(m, l, acc, x_acc[wave], x_ml[wave], lane);
   __syncthreads();
   if (wave != 0) return;
-  merge_and_write<T, G, NW>(I, u, partition, x_acc, x_ml, lane);
+  merge_and_write<T, G, NW>(I, u, partition, x_acc, x_ml, n_active, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -759,6 +769,10 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
   const int hq0 = u.wh * G;
   const int hk = hq0 / I.ratio;
   const int t1 = u.t1;
+
+  // A wave without tokens leaves at once (see the kernel above).
+  if (u.t0 + kGqaTile * wave >= t1) return;
+  const int n_active = min(NW, (t1 - u.t0 + kGqaTile - 1) / kGqaTile);
 
   const int h = lane & 15;               // this lane's head (columns >= G are padding)
   const int g = lane >> 4;               // which 8 of an operand's 32 k-slots
@@ -937,7 +951,7 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
     }
   }
   __syncthreads();
-  merge_and_write_group<T, G, NW>(I, u, partition, x_acc, x_ml, &arrival, lane, wave);
+  merge_and_write_group<T, G, NW>(I, u, partition, x_acc, x_ml, &arrival, n_active, lane, wave);
 }
 
 // Zero-fills the arrival counters (a kernel rather than a memset node so the
