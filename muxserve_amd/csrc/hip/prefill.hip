@@ -76,11 +76,24 @@ struct PrefillParams {
   int32_t out_rows_16b;   // out and its row stride allow 16-byte stores
 };
 
-template <typename T>
+// DMA = true: K and V tiles go from global memory straight into LDS
+// (global_load_lds_dwordx4: lane l's 16 bytes land at base + 16 l), row-major
+// [key][128 dims] with the 16-byte chunks of a row XOR-swizzled by the row
+// number so that fragment reads spread over the banks; V^T fragments come out of
+// the row-major tile with the transposing read ds_read_b64_tr_b16.  No staging
+// registers, no LDS stores, no byte permutes; two tile buffers, one barrier per
+// tile.  DMA = false: the tiles are staged through registers, V transposed on
+// its way into LDS (kept for reference and comparison).
+typedef short v4i16 __attribute__((ext_vector_type(4)));
+constexpr int kTileElems = kBN * kHeadSize;          // one unpadded row-major tile
+
+template <typename T, bool DMA>
 __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillParams P) {
   constexpr int D = kHeadSize;
-  // One buffer: the K tile, then the V^T tile; the epilogue reuses all of it.
-  __shared__ __attribute__((aligned(16))) uint16_t smem[kBN * kKRow + D * kVRow];
+  // DMA: K[2], V[2] tile buffers.  Otherwise one buffer: the K tile, then the
+  // V^T tile.  The epilogue reuses the memory for the output rows.
+  constexpr int kSmemElems = DMA ? 4 * kTileElems : kBN * kKRow + D * kVRow;
+  __shared__ __attribute__((aligned(16))) uint16_t smem[kSmemElems];
   uint16_t *const Ks = smem;
   uint16_t *const Vt = smem + kBN * kKRow;
 
@@ -130,28 +143,42 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
   const int kv_end = min(len, q0 + kBM);
   const int n_tiles = (kv_end + kBN - 1) / kBN;
 
-  // Global -> register staging of one K/V tile.  K: thread takes chunk
-  // (key = tid/16 + 16 i, dchunk = tid%16).  V: thread takes keys 4 kg .. 4 kg+3
-  // (kg = tid%16) of dchunk vc = tid/16.  Addresses are a uniform base plus a
-  // 32-bit per-thread byte offset that advances by one tile per load.  Rows past
-  // the prompt re-read its last row: finite data whose probability is exactly 0
-  // (such a key is in the future of every valid query).
-  const int kc = tid & 15, kk = tid >> 4;
-  const int vg = tid & 15, vc = tid >> 4;
+  // ---- tile staging -------------------------------------------------------------------
   const uint32_t row_bytes = static_cast<uint32_t>(P.kv_stride) * 2u;
   const char *kbase = reinterpret_cast<const char *>(P.k + static_cast<int64_t>(seq_begin) * P.kv_stride + hk * D);
   const char *vbase = reinterpret_cast<const char *>(P.v + static_cast<int64_t>(seq_begin) * P.kv_stride + hk * D);
-  uint32_t koff[4], voff[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    koff[i] = static_cast<uint32_t>(kk + 16 * i) * row_bytes + 16u * kc;
-    voff[i] = static_cast<uint32_t>(4 * vg + i) * row_bytes + 16u * vc;
-  }
   const uint32_t tile_bytes = kBN * row_bytes;
   const uint32_t last_row = static_cast<uint32_t>(len - 1) * row_bytes;
-  const uint32_t kmax = last_row + 16u * kc, vmax = last_row + 16u * vc;
-  u32x4 kst[4], vst[4];
-  auto load_tile = [&]() {                 // loads the next tile in sequence
+  // Rows past the prompt re-read its last row: finite data whose probability is
+  // exactly 0 (such a key is in the future of every valid query).
+
+  // Register path.  K: thread takes chunk (key = tid/16 + 16 i, dchunk = tid%16).
+  // V: thread takes keys 4 kg .. 4 kg+3 (kg = tid%16) of dchunk vc = tid/16.
+  const int kc = tid & 15, kk = tid >> 4;
+  const int vg = tid & 15, vc = tid >> 4;
+  uint32_t koff[4], voff[DMA ? 1 : 4];
+  u32x4 kst[DMA ? 1 : 4], vst[DMA ? 1 : 4];
+  uint32_t kmax, vmax;
+  if constexpr (!DMA) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      koff[i] = static_cast<uint32_t>(kk + 16 * i) * row_bytes + 16u * kc;
+      voff[i] = static_cast<uint32_t>(4 * vg + i) * row_bytes + 16u * vc;
+    }
+    kmax = last_row + 16u * kc;
+    vmax = last_row + 16u * vc;
+  } else {
+    // DMA path.  Instruction i of wave w fills KiB 4 i + w of a tile = rows
+    // 16 i + 4 w .. +3; lane l sits at row 16 i + 4 w + l/16, position l%16, and
+    // fetches chunk position ^ (row % 16) - the same chunk for every i.
+    const int row0 = 4 * wave + (lane >> 4);
+    const int chunk = (lane & 15) ^ (row0 & 15);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) koff[i] = static_cast<uint32_t>(row0 + 16 * i) * row_bytes + 16u * chunk;
+    kmax = last_row + 16u * chunk;
+    vmax = kmax;
+  }
+  auto load_tile = [&]() {                 // register path: loads the next tile in sequence
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       kst[i] = *reinterpret_cast<const u32x4 *>(kbase + min(koff[i], kmax));
@@ -183,15 +210,41 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
       *reinterpret_cast<u32x2 *>(&Vt[(8 * vc + 2 * w + 1) * kVRow + 4 * vg]) = u32x2{hi01, hi23};
     }
   };
+  auto dma_tile = [&](int buf) {           // DMA path: the next tile in sequence into buffer buf
+    typedef __attribute__((address_space(3))) void lds_void;
+    typedef const __attribute__((address_space(1))) void global_void;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t o = min(koff[i], kmax);
+      uint16_t *kd = smem + buf * kTileElems + (4 * i + wave) * 512;
+      uint16_t *vd = smem + (2 + buf) * kTileElems + (4 * i + wave) * 512;
+      // (address-space casts need the C form)
+      __builtin_amdgcn_global_load_lds((global_void *)(kbase + o), (lds_void *)kd, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_void *)(vbase + o), (lds_void *)vd, 16, 0, 0);
+      koff[i] += tile_bytes;
+    }
+  };
 
-  load_tile();
+  if constexpr (DMA) dma_tile(0);
+  else load_tile();
   for (int t = 0; t < n_tiles; ++t) {
     const int k0 = t * kBN;
-    __syncthreads();                     // everyone is done reading the previous tile
-    store_tile();
-    __syncthreads();
-    if (t + 1 < n_tiles) load_tile();
+    const int cur = t & 1;
+    if constexpr (DMA) {
+      // This wave's part of tile t has landed; after the barrier all of it has,
+      // and everybody is done with the other buffer.
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (t + 1 < n_tiles) dma_tile(cur ^ 1);
+    } else {
+      __syncthreads();                     // everyone is done reading the previous tile
+      store_tile();
+      __syncthreads();
+      if (t + 1 < n_tiles) load_tile();
+    }
     if (k0 > wq0 + 31) continue;         // every key of the tile is in this wave's future
+    const uint16_t *const Kt = DMA ? smem + cur * kTileElems : Ks;           // this tile's K
+    const uint16_t *const Vr = DMA ? smem + (2 + cur) * kTileElems : Vt;     // this tile's V (row-major) or V^T
 
     // ---- S^T = K . Q^T : two 32-key blocks ------------------------------------------
     // LDS fragment reads run kDepth steps ahead of the MFMAs that consume them.
@@ -204,19 +257,25 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
 #pragma unroll
       for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
     {
-      const uint16_t *kr = &Ks[qcol * kKRow + 8 * half];
+      // Fragment j: key block j % 2, dims 16 (j / 2) + 8 half .. +7 of key row qcol.
+      auto read_k = [&](int j) {
+        Frag f;
+        if constexpr (DMA) {
+          const int row = 32 * (j % 2) + qcol, chunk = 2 * (j / 2) + half;
+          f.u = *reinterpret_cast<const u32x4 *>(Kt + row * D + 8 * (chunk ^ (row & 15)));
+        } else {
+          f.u = *reinterpret_cast<const u32x4 *>(Kt + (32 * (j % 2) + qcol) * kKRow + 16 * (j / 2) + 8 * half);
+        }
+        return f;
+      };
       Frag ring[kDepth];
 #pragma unroll
-      for (int j = 0; j < kDepth; ++j)
-        ring[j].u = *reinterpret_cast<const u32x4 *>(kr + (j % 2) * 32 * kKRow + 16 * (j / 2));
+      for (int j = 0; j < kDepth; ++j) ring[j] = read_k(j);
       __builtin_amdgcn_sched_barrier(0);   // keep the scheduler from sinking the reads to their uses
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         sacc[j % 2] = mfma<T>(ring[j % kDepth], qf[j / 2], sacc[j % 2]);
-        if (j + kDepth < 16) {
-          const int n = j + kDepth;
-          ring[j % kDepth].u = *reinterpret_cast<const u32x4 *>(kr + (n % 2) * 32 * kKRow + 16 * (n / 2));
-        }
+        if (j + kDepth < 16) ring[j % kDepth] = read_k(j + kDepth);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -292,13 +351,34 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
     // ---- O^T += V^T . P^T ---------------------------------------------------------------
     // k-slot j of lane half h in step (kb, st) is key 32 kb + 16 st + 8 (j/4) + 4 h + j%4
     {
-      const uint16_t *vr = &Vt[qcol * kVRow + 4 * half];
       auto read_v = [&](int n) {         // fragment n = 4 ks + mb
-        const uint16_t *r = vr + (n % 4) * 32 * kVRow + 16 * (n / 4);
-        const u32x2 lo = *reinterpret_cast<const u32x2 *>(r);
-        const u32x2 hi = *reinterpret_cast<const u32x2 *>(r + 8);
+        const int mb = n % 4, ks = n / 4;
         Frag f;
-        f.u = u32x4{lo.x, lo.y, hi.x, hi.y};
+        if constexpr (DMA) {
+          // The transposing read works on groups of 16 lanes: lane 4 j + m of a
+          // group points at dims 4 m .. 4 m + 3 of key row j, and lane i of the
+          // group receives dim i of rows 0..3.  Here a group covers dims
+          // 32 mb + 16 (lane/16 % 2) .. +15 and keys 16 ks + 4 half (+ 8) .. +3.
+          typedef __attribute__((address_space(3))) v4i16 lds_v4i16;
+          const int jrow = (lane & 15) >> 2, m = lane & 3;
+          const int chunk = 4 * mb + 2 * ((lane >> 4) & 1) + (m >> 1);
+          u32x2 part[2];
+#pragma unroll
+          for (int hsel = 0; hsel < 2; ++hsel) {
+            const int row = 16 * ks + 8 * hsel + 4 * half + jrow;
+            const uint16_t *src = Vr + row * D + 8 * (chunk ^ (row & 15)) + 4 * (m & 1);
+            const v4i16 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16 *)src);
+            union { v4i16 v; u32x2 u; } c;
+            c.v = r;
+            part[hsel] = c.u;
+          }
+          f.u = u32x4{part[0].x, part[0].y, part[1].x, part[1].y};
+        } else {
+          const uint16_t *r = Vr + (32 * mb + qcol) * kVRow + 4 * half + 16 * ks;
+          const u32x2 lo = *reinterpret_cast<const u32x2 *>(r);
+          const u32x2 hi = *reinterpret_cast<const u32x2 *>(r + 8);
+          f.u = u32x4{lo.x, lo.y, hi.x, hi.y};
+        }
         return f;
       };
       Frag ring[kDepth];
@@ -323,7 +403,7 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
     // lane, four rows per instruction) instead of 8-byte pieces of 32 rows: the
     // tile buffers are free once every wave has left the loop.
     constexpr int kORow = D + 8;         // 272-byte rows
-    static_assert(4 * 32 * kORow <= kBN * kKRow + D * kVRow, "output staging fits the tile buffers");
+    static_assert(4 * 32 * kORow <= kSmemElems, "output staging fits the tile buffers");
     __syncthreads();
     uint16_t *stage = smem + wave * 32 * kORow;
 #pragma unroll
@@ -403,8 +483,9 @@ extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const v
   if (n_wg > 0x7fffffff) return MUXA_EUNSUPPORTED;
   const dim3 grid(static_cast<uint32_t>(n_wg));
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (dtype == MUXA_DTYPE_F16) hipLaunchKernelGGL(prefill_causal_kernel<F16>, grid, dim3(256), 0, st, P);
-  else hipLaunchKernelGGL(prefill_causal_kernel<BF16>, grid, dim3(256), 0, st, P);
+  constexpr bool kDma = true;
+  if (dtype == MUXA_DTYPE_F16) hipLaunchKernelGGL((prefill_causal_kernel<F16, kDma>), grid, dim3(256), 0, st, P);
+  else hipLaunchKernelGGL((prefill_causal_kernel<BF16, kDma>), grid, dim3(256), 0, st, P);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e);
   return MUXA_OK;
