@@ -131,7 +131,6 @@ def bench_prefill3(args):
     import torch
     from muxserve_amd import ops, workloads
     from muxserve_amd.pool import HEAD_SIZE as D, allocate_gpu_cache
-    from oracle import attn_oracle as orc
     dev, bs = "cuda:0", 16
     models = workloads.config3(seed=args.seed)
     total_blocks = sum(int(((m.prompt_lens + bs - 1) // bs).sum()) * m.num_kv_heads for m in models)
@@ -150,8 +149,8 @@ def bench_prefill3(args):
         slots, used = workloads.prefill_slot_mapping(m.prompt_lens, Hkv, bs, ids[cur:])
         cur += used
         work.append((m, q, k, v, out, cu, torch.from_numpy(slots).to(dev), T))
-        flops += 4.0 * Hq * D * float((m.prompt_lens.astype(np.float64) * (m.prompt_lens + 1) / 2).sum())
-        wbytes += orc.cache_write_bytes(T, Hkv)
+        flops += workloads.prefill_flops(m.prompt_lens, Hq)
+        wbytes += workloads.cache_write_bytes(T, Hkv)
         tokens += T
 
     def attn(_):
@@ -162,31 +161,14 @@ def bench_prefill3(args):
         for m, q, k, v, out, cu, slots, T in work:
             ops.reshape_and_cache(k, v, k_pool, v_pool, slots, num_tokens=T)
 
-    # The same three launches as three colocated jobs: one stream per model, all
-    # started together, the step ends when the last one does.
-    streams = [torch.cuda.Stream() for _ in work]
-    main = torch.cuda.current_stream()
-
-    def attn_colocated(_):
-        start = torch.cuda.Event()
-        start.record(main)
-        for st, (m, q, k, v, out, cu, slots, T) in zip(streams, work):
-            st.wait_event(start)
-            ops.prefill_causal(out, q, k, v, cu, int(m.prompt_lens.max()), m.scale, m.num_kv_heads, stream=st)
-            done = torch.cuda.Event()
-            done.record(st)
-            main.wait_event(done)
-
     ms_a = _time(attn, args.steps, args.warmup)
-    ms_c = _time(attn_colocated, args.steps, args.warmup)
     ms_w = _time(write, args.steps, args.warmup)
     tf = flops / (ms_a * 1e-3) / 1e12
     gbs = wbytes / (ms_w * 1e-3) / 1e9
     cfg = {"workload": "prefill3", "prompts_per_model": 16, "tokens": tokens, "flops": flops,
-           "three_streams_ms": ms_c, "three_streams_tflops": flops / (ms_c * 1e-3) / 1e12,
            "cache_write_ms": ms_w, "cache_write_gbs": gbs, "cache_write_frac_of_hbm": gbs / HBM_PEAK_GBS}
     roof = {"bound": "mfma", "achieved": tf, "peak": 2500.0, "unit": "TFLOP/s", "frac": tf / 2500.0,
-            "traffic": None, "kernel": "prefill_causal_kernel<F16>"}
+            "traffic": None, "kernel": "prefill_causal_kernel<F16,true>"}
     return _line("prefill causal attention tokens/s (3 models, 16 prompts each)", tokens / (ms_a * 1e-3),
                  "tokens/s", args, ms_a, cfg, roof)
 
@@ -197,7 +179,6 @@ def bench_cache_write(args):
     import torch
     from muxserve_amd import ops, workloads
     from muxserve_amd.pool import HEAD_SIZE as D, allocate_gpu_cache
-    from oracle import attn_oracle as orc
     dev, bs = "cuda:0", 16
     N = 1 << 20
     k_pool, v_pool = allocate_gpu_cache(N, bs, dev)
@@ -212,7 +193,7 @@ def bench_cache_write(args):
         dec.append((kv[:, :hk * D], kv[:, hk * D:], torch.from_numpy(slots).to(dev), b, hk))
     ms_d = _time(lambda _: [ops.reshape_and_cache(k, v, k_pool, v_pool, s) for k, v, s, b, hk in dec],
                  args.steps, args.warmup)
-    bytes_d = sum(orc.cache_write_bytes(b, hk) for *_, b, hk in dec)
+    bytes_d = sum(workloads.cache_write_bytes(b, hk) for *_, b, hk in dec)
     # prefill-shaped
     lens = np.full(4, 1024)
     slots, _ = workloads.prefill_slot_mapping(lens, 52, bs, rng.permutation(N))
@@ -221,7 +202,7 @@ def bench_cache_write(args):
     dslots = torch.from_numpy(slots).to(dev)
     ms_p = _time(lambda _: ops.reshape_and_cache(kv[:, :52 * D], kv[:, 52 * D:], k_pool, v_pool, dslots),
                  args.steps, args.warmup)
-    bytes_p = orc.cache_write_bytes(T, 52)
+    bytes_p = workloads.cache_write_bytes(T, 52)
     gbs = bytes_p / (ms_p * 1e-3) / 1e9
     cfg = {"workload": "cache_write", "prefill_shape": "52 heads x 4096 tokens", "prefill_bytes": bytes_p,
            "decode_shape": "7b/13b/30b, 56 tokens, three launches", "decode_ms": ms_d, "decode_bytes": bytes_d,
@@ -240,7 +221,6 @@ def bench_colocated(args):
     import torch
     from muxserve_amd import ops, workloads
     from muxserve_amd.pool import HEAD_SIZE as D, allocate_gpu_cache, num_gpu_blocks
-    from oracle import attn_oracle as orc
     dev, bs = "cuda:0", 16
     N = num_gpu_blocks(args.pool_util, torch.cuda.get_device_properties(0).total_memory, bs)
     k_pool, v_pool = allocate_gpu_cache(N, bs, dev)
@@ -254,7 +234,7 @@ def bench_colocated(args):
         bt, _ = workloads.build_tables(ctx, 32, bs, rng.choice(N, size=need, replace=False))
         m = workloads.DecodeModel("7b", 32, 32, ctx, bt).to_device(dev, torch.float16, seed=i)
         dsets.append(m)
-    dbytes = float(np.mean([orc.decode_bytes(m.context_lens, 32, 32, bs) for m in dsets]))
+    dbytes = float(np.mean([workloads.decode_bytes(m.context_lens, 32, 32, bs) for m in dsets]))
     # prefill: 30B shape, 4 prompts x 1024 tokens
     T = 4096
     qkv = torch.randn((T, 3 * 52 * D), generator=g).half().to(dev)
@@ -309,7 +289,6 @@ def bench_gqa_long(args):
     import torch
     from muxserve_amd import ops, workloads
     from muxserve_amd.pool import allocate_gpu_cache
-    from oracle import attn_oracle as orc
     dev, bs = "cuda:0", 16
     N = int(200e9) // 8192 // 128 * 128
     k_pool, v_pool = allocate_gpu_cache(N, bs, dev, dtype=torch.bfloat16)
@@ -324,7 +303,7 @@ def bench_gqa_long(args):
                          m.scale, partition_size=args.partition, total_context_len=int(m.context_lens.sum()))
 
     ms = _time(step, args.steps, args.warmup)
-    nbytes = float(np.mean([orc.decode_bytes(m.context_lens, 64, 8, bs) for m in sets]))
+    nbytes = float(np.mean([workloads.decode_bytes(m.context_lens, 64, 8, bs) for m in sets]))
     gbs = nbytes / (ms * 1e-3) / 1e9
     cfg = {"workload": "gqa_long", "shape": "Hq64/Hkv8, B=64, ctx U[2048,8192], bf16", "pool_gb": round(N * 8192 / 1e9, 1),
            "bytes_per_step": int(nbytes), "partition": args.partition}
@@ -351,7 +330,6 @@ def main():
     import torch
     from muxserve_amd import ops, workloads
     from muxserve_amd.pool import allocate_gpu_cache, num_gpu_blocks
-    from oracle import attn_oracle as orc   # traffic formula + cpu baseline only
 
     dev = "cuda:0"
     bs = 16
@@ -401,7 +379,7 @@ def main():
     ms = max(wall_ms, ev_ms)
 
     tokens = sum(m.batch for m in sets[0][0])
-    step_bytes = [sum(orc.decode_bytes(m.context_lens, m.num_q_heads, m.num_kv_heads, bs) for m in models)
+    step_bytes = [sum(workloads.decode_bytes(m.context_lens, m.num_q_heads, m.num_kv_heads, bs) for m in models)
                   for models, _ in sets]
     visits = [len(range(i, args.steps, len(sets))) for i in range(len(sets))]
     avg_bytes = sum(b * v for b, v in zip(step_bytes, visits)) / max(1, sum(visits))

@@ -216,3 +216,28 @@ def prefill_slot_mapping(prompt_lens, num_kv_heads, block_size, ids):
         i = np.arange(n)
         rows.append(blk[i // block_size] * block_size + (i % block_size)[:, None])
     return np.concatenate(rows)[:, None, :].astype(np.int64), cur
+
+
+# ---- algorithmic traffic and work (the figures throughput is priced in) ----------
+
+def decode_bytes(context_lens, num_q_heads, num_kv_heads, block_size, head_size=HEAD_SIZE, e=2):
+    """Bytes one decode step of one layer has to move: K and V of exactly the
+    valid tokens, q read and output written, the block-table entries in use and
+    the context length of every sequence."""
+    ctx = np.asarray(context_lens, dtype=np.int64)
+    kv = 2 * ctx * num_kv_heads * head_size * e
+    qo = 2 * num_q_heads * head_size * e
+    table = num_kv_heads * ((ctx + block_size - 1) // block_size) * 4 + 4
+    return int((kv + qo + table).sum())
+
+
+def cache_write_bytes(num_tokens, num_kv_heads, head_size=HEAD_SIZE, e=2):
+    """k and v read, the same bytes written to the pool, one 8-byte slot per
+    (token, head)."""
+    return int(num_tokens) * num_kv_heads * (4 * head_size * e + 8)
+
+
+def prefill_flops(prompt_lens, num_q_heads, head_size=HEAD_SIZE):
+    """QK^T and PV over the causal triangle: 4 * Hq * D * sum L (L + 1) / 2."""
+    lens = np.asarray(prompt_lens, dtype=np.float64)
+    return 4.0 * num_q_heads * head_size * float((lens * (lens + 1) / 2).sum())

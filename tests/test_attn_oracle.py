@@ -234,3 +234,18 @@ def test_rotary_oracle_is_a_complex_rotation():
         rb, _ = orc.rotary_neox(torch.tensor([n]), b, b)
         return float((ra * rb).sum())
     assert abs(dot(5, 2) - dot(103, 100)) < 1e-3 and abs(dot(5, 2) - dot(6, 2)) > 1e-4
+
+
+def test_traffic_formulas_of_the_package_agree_with_the_oracle():
+    """bench.py prices throughput with muxserve_amd.workloads' formulas; the
+    oracle holds its own statement of the same definitions."""
+    from muxserve_amd import workloads
+    rng = np.random.Generator(np.random.PCG64(5))
+    for Hq, Hkv, bs in ((32, 32, 16), (64, 8, 16), (40, 40, 8), (52, 52, 32)):
+        ctx = rng.integers(1, 3000, size=37)
+        assert workloads.decode_bytes(ctx, Hq, Hkv, bs) == orc.decode_bytes(ctx, Hq, Hkv, bs)
+        assert workloads.cache_write_bytes(int(ctx.sum()), Hkv) == orc.cache_write_bytes(int(ctx.sum()), Hkv)
+    # one sequence by hand: 100 tokens, 2 kv heads, 4 q heads, 16-token blocks
+    assert workloads.decode_bytes([100], 4, 2, 16) == 2 * 100 * 2 * 128 * 2 + 2 * 4 * 128 * 2 + 2 * 7 * 4 + 4
+    assert workloads.cache_write_bytes(3, 2) == 3 * 2 * 1032
+    assert workloads.prefill_flops([1, 3], 2) == 4.0 * 2 * 128 * (1 + 6)
