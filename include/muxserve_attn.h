@@ -188,6 +188,43 @@ int32_t mux_rope_reshape_and_cache(const int64_t *positions, void *q, int64_t q_
                                    int32_t num_kv_heads, int32_t head_size, int32_t block_size,
                                    int32_t dtype, void *stream);
 
+/* ---- Operators of the model step around the attention layer ---------------
+ * The reference's LLaMA layer takes RMSNorm and SiluAndMul from its vLLM fork
+ * (muxserve/flexserver/models/llama.py:35-36; used at :79-81, 200-203, 217-232,
+ * 257, 283) and samples with its own GreedySampler
+ * (muxserve/flexserver/sampler.py:9-35).  Device pointers, row strides in
+ * elements; rows and weights 16-byte aligned, sizes multiples of 8.
+ *
+ * mux_rms_norm: out[t,:] = T(x[t,:] * rsqrt(mean(x[t,:]^2) + eps)) * weight,
+ * statistics in fp32, the product with the weight taken in the storage type T. */
+int32_t mux_rms_norm(void *out, int64_t out_row_stride, const void *x, int64_t x_row_stride,
+                     const void *weight, float eps, int32_t num_tokens, int32_t hidden_size,
+                     int32_t dtype, void *stream);
+
+/* mux_silu_and_mul: x [num_tokens, 2 d] = [gate | up] ->
+ * out[t,:] = T(gate / (1 + exp(-gate))) * up, the product taken in T. */
+int32_t mux_silu_and_mul(void *out, int64_t out_row_stride, const void *x, int64_t x_row_stride,
+                         int32_t num_tokens, int32_t d, int32_t dtype, void *stream);
+
+/* mux_greedy_sample: GreedySampler.forward (sampler.py:15-35) without
+ * materialising the logits.  For sampled row r < num_rows:
+ *     h = hidden_states[row_index ? row_index[r] : r]
+ *     next_tokens[r] = argmax_{v < vocab_size} T(h . embedding[v,:])
+ * (fp32 accumulation, each logit rounded to T before the comparison as the
+ * reference's fp16 logits are; ties go to the lowest id).  On a prompt step
+ * row_index holds cumsum(prompt_lens) - 1 (sampler.py:18-24), on a decode step
+ * it is NULL.  embedding: [embedding_rows >= vocab_size, hidden_size], the
+ * lm_head weight (models/llama.py:317-323); hidden_size a multiple of 256.
+ * next_tokens: DEVICE int64 [num_rows].  workspace: DEVICE,
+ * mux_greedy_sample_workspace_bytes(vocab_size) bytes, 16-byte aligned, no
+ * initialisation needed; calls that share it must not overlap. */
+size_t mux_greedy_sample_workspace_bytes(int32_t vocab_size);
+int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_states, int64_t hidden_row_stride,
+                          const int32_t *row_index, int32_t num_rows, const void *embedding,
+                          int64_t embedding_row_stride, int32_t embedding_rows, int32_t vocab_size,
+                          int32_t hidden_size, int32_t dtype, void *workspace, size_t workspace_bytes,
+                          void *stream);
+
 /* ---- CU-masked streams ---------------------------------------------------
  * Replacement for the reference's per-process MPS share
  * (CUDA_MPS_ACTIVE_THREAD_PERCENTAGE, muxserve/muxsched/launcher.py:54-61):

@@ -129,6 +129,11 @@ ATTN_SIGNATURES = {
                                 c_i32, c_vp]),
     "mux_rope_reshape_and_cache": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i32, c_i32, c_vp, c_vp, c_i64,
                                            c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp]),
+    "mux_rms_norm": (c_i32, [c_vp, c_i64, c_vp, c_i64, c_vp, c_f32, c_i32, c_i32, c_i32, c_vp]),
+    "mux_silu_and_mul": (c_i32, [c_vp, c_i64, c_vp, c_i64, c_i32, c_i32, c_i32, c_vp]),
+    "mux_greedy_sample_workspace_bytes": (c_sz, [c_i32]),
+    "mux_greedy_sample": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_i32, c_vp, c_i64, c_i32, c_i32, c_i32, c_i32,
+                                  c_vp, c_sz, c_vp]),
     "mux_stream_create_cu_range": (c_i32, [c_vp, c_i32, c_i32, c_vp]),
     "mux_stream_destroy": (c_i32, [c_vp]),
     "mux_device_cu_info": (c_i32, [c_vp]),

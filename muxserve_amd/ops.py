@@ -246,6 +246,86 @@ def rope_reshape_and_cache(positions: torch.Tensor, q: Optional[torch.Tensor], k
     _lib.check_attn(rc, "mux_rope_reshape_and_cache")
 
 
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None,
+             num_tokens: Optional[int] = None, stream=None) -> torch.Tensor:
+    """out[t] = T(x[t] * rsqrt(mean(x[t]^2) + eps)) * weight for x [T, hidden]."""
+    _need_cuda(x, weight)
+    if out is None:
+        out = torch.empty_like(x)
+    _need_cuda(out)
+    if weight.dim() != 1 or weight.shape[0] != x.shape[1] or weight.dtype != x.dtype or not weight.is_contiguous():
+        raise ValueError("weight: expected contiguous [hidden] of the dtype of x")
+    if out.shape != x.shape or out.dtype != x.dtype:
+        raise ValueError("out: expected the shape and dtype of x")
+    T = x.shape[0] if num_tokens is None else min(int(num_tokens), x.shape[0])
+    rc = _lib.attn().mux_rms_norm(out.data_ptr(), _rows(out, "out"), x.data_ptr(), _rows(x, "x"), weight.data_ptr(),
+                                  float(eps), T, x.shape[1], _dtype_code(x), _stream_ptr(stream))
+    _lib.check_attn(rc, "mux_rms_norm")
+    return out
+
+
+def silu_and_mul(x: torch.Tensor, out: Optional[torch.Tensor] = None, num_tokens: Optional[int] = None,
+                 stream=None) -> torch.Tensor:
+    """x [T, 2 d] = [gate | up] -> out [T, d] = silu(gate) * up."""
+    _need_cuda(x)
+    if x.dim() != 2 or x.shape[1] % 2:
+        raise ValueError("x: expected [T, 2 d]")
+    d = x.shape[1] // 2
+    if out is None:
+        out = torch.empty((x.shape[0], d), dtype=x.dtype, device=x.device)
+    _need_cuda(out)
+    if tuple(out.shape) != (x.shape[0], d) or out.dtype != x.dtype:
+        raise ValueError("out: expected [T, d] of the dtype of x")
+    T = x.shape[0] if num_tokens is None else min(int(num_tokens), x.shape[0])
+    rc = _lib.attn().mux_silu_and_mul(out.data_ptr(), _rows(out, "out"), x.data_ptr(), _rows(x, "x"), T, d,
+                                      _dtype_code(x), _stream_ptr(stream))
+    _lib.check_attn(rc, "mux_silu_and_mul")
+    return out
+
+
+_sample_workspaces = {}
+
+
+def greedy_sample(embedding: torch.Tensor, hidden_states: torch.Tensor, vocab_size: int, num_rows: int,
+                  row_index: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                  workspace: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
+    """int64 [num_rows] on the device: argmax over v < vocab_size of
+    hidden_states[row] . embedding[v], row = row_index[r] (int32, device) or r."""
+    _need_cuda(embedding, hidden_states)
+    if embedding.dim() != 2 or hidden_states.dim() != 2 or embedding.shape[1] != hidden_states.shape[1]:
+        raise ValueError("embedding [V, hidden] and hidden_states [T, hidden] expected")
+    if embedding.dtype != hidden_states.dtype:
+        raise TypeError("embedding and hidden_states dtypes differ")
+    num_rows = int(num_rows)
+    ri_ptr = None
+    if row_index is not None:
+        _need_cuda(row_index)
+        if row_index.dtype != torch.int32 or row_index.dim() != 1 or not row_index.is_contiguous() \
+                or row_index.shape[0] < num_rows:
+            raise ValueError("row_index: expected contiguous int32 [>= num_rows]")
+        ri_ptr = row_index.data_ptr()
+    elif hidden_states.shape[0] < num_rows:
+        raise ValueError("fewer rows of hidden states than sampled rows")
+    if out is None:
+        out = torch.empty((num_rows,), dtype=torch.int64, device=hidden_states.device)
+    if out.dtype != torch.int64 or out.dim() != 1 or out.shape[0] < num_rows or not out.is_contiguous():
+        raise ValueError("out: expected contiguous int64 [>= num_rows]")
+    lib = _lib.attn()
+    need = lib.mux_greedy_sample_workspace_bytes(int(vocab_size))
+    if workspace is None:
+        key = (hidden_states.device, torch.cuda.current_stream(hidden_states.device).cuda_stream)
+        workspace = _sample_workspaces.get(key)
+        if workspace is None or workspace.numel() < need:
+            workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=hidden_states.device)
+            _sample_workspaces[key] = workspace
+    rc = lib.mux_greedy_sample(out.data_ptr(), hidden_states.data_ptr(), _rows(hidden_states, "hidden_states"), ri_ptr,
+                               num_rows, embedding.data_ptr(), _rows(embedding, "embedding"), embedding.shape[0],
+                               int(vocab_size), hidden_states.shape[1], _dtype_code(hidden_states),
+                               workspace.data_ptr(), workspace.numel(), _stream_ptr(stream))
+    _lib.check_attn(rc, "mux_greedy_sample")
+    return out[:num_rows]
+
+
 class CUMaskedStream:
     """A HIP stream restricted to a share of the GPU's compute units (the
     replacement for a per-process MPS percentage).  Usable wherever a stream is
