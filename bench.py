@@ -54,7 +54,7 @@ def parse():
     ap.add_argument("--no-hint", action="store_true", help="do not pass the host-side sum of context lengths")
     ap.add_argument("--unfused", action="store_true", help="one launch per model instead of one fused launch")
     ap.add_argument("--workload", default="mixed3_decode",
-                    choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long"],
+                    choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long", "model_ops"],
                     help="mixed3_decode is the headline metric; the others are the remaining synthetic "
                          "shapes, each printing its own JSON line")
     return ap.parse_args()
@@ -315,6 +315,66 @@ def bench_gqa_long(args):
     return _line("long-context GQA decode attn tokens/s", 64 / (ms * 1e-3), "tokens/s", args, ms, cfg, roof, dtype="bf16")
 
 
+def bench_model_ops(args):
+    """The per-step operators around the attention layer: greedy sampling
+    (lm_head + argmax in one pass) for the three models of the mix, RMSNorm and
+    SiluAndMul on a prefill-sized step of the 30B shape."""
+    import torch
+    import torch.nn.functional as F
+    from muxserve_amd import ops
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(args.seed)
+    V = 32000
+    shapes = [("7b", 4096, 32), ("13b", 5120, 16), ("30b", 6656, 8)]
+    heads = []
+    sbytes = 0
+    for name, hidden, R in shapes:
+        emb = (torch.randn((V, hidden), generator=g) * 0.05).half().to(dev)
+        hid = torch.randn(((R + 7) // 8 * 8, hidden), generator=g).half().to(dev)
+        out = torch.empty((R,), dtype=torch.int64, device=dev)
+        heads.append((emb, hid, R, out))
+        sbytes += V * hidden * 2 + R * hidden * 2 + R * 8
+
+    def sample(_):
+        for emb, hid, R, out in heads:
+            ops.greedy_sample(emb, hid, V, R, out=out)
+
+    def sample_torch(_):
+        for emb, hid, R, out in heads:
+            torch.argmax(torch.matmul(hid[:R], emb.t())[:, :V], dim=-1, out=out)
+
+    ms_s = _time(sample, args.steps, args.warmup)
+    ms_st = _time(sample_torch, args.steps, args.warmup)
+
+    T, hidden, d = 4096, 6656, 17920
+    xs = [torch.randn((T, hidden), generator=g).half().to(dev) for _ in range(4)]
+    outs = [torch.empty_like(x) for x in xs]
+    w = (1 + 0.1 * torch.randn((hidden,), generator=g)).half().to(dev)
+    ms_n = _time(lambda i: ops.rms_norm(xs[i % 4], w, 1e-6, out=outs[i % 4]), args.steps, args.warmup)
+    ms_nt = _time(lambda i: F.rms_norm(xs[i % 4], (hidden,), w, 1e-6), args.steps, args.warmup)
+    nbytes = 2 * T * hidden * 2 + hidden * 2
+    del xs, outs
+    gu = [torch.randn((T, 2 * d), generator=g).half().to(dev) for _ in range(2)]
+    go = [torch.empty((T, d), dtype=torch.float16, device=dev) for _ in range(2)]
+    ms_a = _time(lambda i: ops.silu_and_mul(gu[i % 2], out=go[i % 2]), args.steps, args.warmup)
+    ms_at = _time(lambda i: torch.mul(F.silu(gu[i % 2][:, :d]), gu[i % 2][:, d:], out=go[i % 2]), args.steps,
+                  args.warmup)
+    abytes = 3 * T * d * 2
+
+    gbs = sbytes / (ms_s * 1e-3) / 1e9
+    cfg = {"workload": "model_ops",
+           "sampler": "7b(hidden 4096, 32 rows)+13b(5120, 16)+30b(6656, 8), vocabulary 32000, three launches per step",
+           "sampler_bytes_per_step": sbytes, "sampler_torch_matmul_argmax_ms": ms_st,
+           "rms_norm": {"shape": [T, hidden], "ms": ms_n, "gbs": nbytes / (ms_n * 1e-3) / 1e9,
+                        "frac_of_hbm": nbytes / (ms_n * 1e-3) / 1e9 / HBM_PEAK_GBS, "torch_ms": ms_nt},
+           "silu_and_mul": {"shape": [T, 2 * d], "ms": ms_a, "gbs": abytes / (ms_a * 1e-3) / 1e9,
+                            "frac_of_hbm": abytes / (ms_a * 1e-3) / 1e9 / HBM_PEAK_GBS, "torch_ms": ms_at}}
+    roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+            "traffic": None, "kernel": "lm_head_argmax_kernel<F16,NB,KT>"}
+    return _line("greedy sampling tokens/s (lm_head + argmax, 3 models)", 56 / (ms_s * 1e-3), "tokens/s", args, ms_s,
+                 cfg, roof)
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -322,7 +382,7 @@ def main():
               file=sys.stderr)
         sys.exit(2)
     other = {"prefill3": bench_prefill3, "cache_write": bench_cache_write, "colocated": bench_colocated,
-             "gqa_long": bench_gqa_long}
+             "gqa_long": bench_gqa_long, "model_ops": bench_model_ops}
     if args.workload in other:
         print(json.dumps(other[args.workload](args)))
         return

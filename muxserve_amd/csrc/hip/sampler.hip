@@ -4,18 +4,24 @@
 // reads the [vocab, hidden] matrix once (262 MB for a 7B model) and a few rows of
 // hidden states, so the kernel is bound by HBM.
 //
-// lm_head_argmax_kernel<T, NB, KT>: a workgroup owns 64 vocabulary rows (16 per
-// wave) and up to 16 NB sampled rows of hidden states.  It walks the hidden
-// dimension in tiles of KT: the hidden-state tile is staged in LDS (shared by
-// the four waves, double-buffered, one barrier per tile) while every wave
-// streams its 16 embedding rows from global memory straight into MFMA A
-// operands (v_mfma_f32_16x16x32: lane l supplies row l % 16, columns
-// 8 (l / 16) .. +7 of a 32-column slice, i.e. 16 rows x 64 contiguous bytes per
-// load instruction), one tile ahead of its use.  Accumulators hold
-// logits[vocab row 4 (l / 16) + i][sampled row l % 16]; each is rounded to the
-// storage type (the reference compares logits of that type), reduced to the
-// workgroup's (max, lowest index) per sampled row and written to a partial
-// table.  argmax_finish_kernel reduces the table: one wave per sampled row.
+// lm_head_argmax_kernel<T, NB>: a workgroup owns 64 vocabulary rows (16 per
+// wave) and up to 16 NB sampled rows of hidden states, and walks the hidden
+// dimension in tiles of 128.
+//   * Hidden states: the tile [16 NB][128] is staged in LDS, shared by the four
+//     waves, double-buffered, one barrier per tile.
+//   * Embedding rows: the MFMA A operand wants lane l to hold row l % 16
+//     (v_mfma_f32_16x16x32: columns 8 (l / 16) .. +7 of a 32-column slice) -
+//     loaded that way, every 16 lanes would touch 16 different rows with 16 bytes
+//     each.  Instead a load instruction takes 4 rows x 256 contiguous bytes
+//     (16 lanes per row), two tiles ahead of their use, and the wave regroups
+//     its 4 KiB tile through a private LDS area: 16-byte chunk c of row r sits at
+//     position c ^ r of the row, so both the row-wise writes and the
+//     column-wise fragment reads are free of bank conflicts.
+// Accumulators hold logits[vocab row 4 (l / 16) + i][sampled row l % 16]; each is
+// rounded to the storage type (the reference compares logits of that type),
+// reduced to the workgroup's (max, lowest index) per sampled row and written to
+// a partial table.  argmax_finish_kernel reduces the table: one wave per
+// sampled row.
 #include "mux_common.h"
 
 namespace mux {
@@ -59,16 +65,16 @@ __device__ __forceinline__ void take_better(float &v, int &i, float ov, int oi) 
   }
 }
 
-// KT = hidden elements per LDS tile (256, or 128 when 64 sampled rows are held,
-// so that two tile buffers stay at 34 KB).
-template <typename T, int NB, int KT>
+template <typename T, int NB>
 __global__ __launch_bounds__(256) void lm_head_argmax_kernel(const LmHeadParams P) {
+  constexpr int KT = 128;                             // hidden elements per tile
   constexpr int ROWS = 16 * NB;                       // sampled rows held in LDS
-  constexpr int CPR = KT / 8;                         // 16-byte chunks per tile row
-  constexpr int SJ = ROWS * CPR / 256;                // staging chunks per thread
-  constexpr int NF = KT / 32;                         // MFMA column slices per tile
-  constexpr int kSmRow = KT + 8;    // LDS row pitch: 16 bytes of padding keep b128 reads off each other's banks
-  __shared__ __attribute__((aligned(16))) uint16_t tile[2][ROWS * kSmRow];
+  constexpr int CPR = KT / 8;                         // 16-byte chunks per tile row (16)
+  constexpr int SJ = ROWS * CPR / 256;                // hidden-state staging chunks per thread (= NB)
+  constexpr int NF = KT / 32;                         // MFMA column slices per tile (4)
+  constexpr int kHRow = KT + 8;     // LDS row pitch: 16 bytes of padding keep b128 reads off each other's banks
+  __shared__ __attribute__((aligned(16))) uint16_t htile[2][ROWS * kHRow];
+  __shared__ __attribute__((aligned(16))) uint16_t wtile[4][16 * KT];      // one 4 KiB area per wave
   __shared__ float red_v[4][ROWS];
   __shared__ int red_i[4][ROWS];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -76,24 +82,29 @@ __global__ __launch_bounds__(256) void lm_head_argmax_kernel(const LmHeadParams 
   const int n_tiles = P.hidden_size / KT;
 
   // Embedding rows of this wave (rows past the vocabulary re-read its last row
-  // and are masked at the end).
+  // and are masked at the end).  Load instruction j: lane l takes row
+  // 4 j + l / 16, and of that row the chunk (l % 16) ^ row.
   const int vrow0 = blockIdx.x * kSmVocabPerWg + 16 * wave;
-  const int lrow = min(vrow0 + r16, P.vocab - 1);
-  const uint16_t *wp = P.weight + static_cast<int64_t>(lrow) * P.weight_stride + 8 * g;
+  const uint16_t *wsrc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = 4 * j + g;
+    const int lrow = min(vrow0 + row, P.vocab - 1);
+    wsrc[j] = P.weight + static_cast<int64_t>(lrow) * P.weight_stride + 8 * (r16 ^ row);
+  }
+  uint16_t *const wmine = &wtile[wave][0];
 
-  // Hidden-state staging: chunk id = tid + 256 j -> (row id / CPR, 16-byte chunk id % CPR).
+  // Hidden-state staging: chunk id = tid + 256 j -> (row id / 16, 16-byte chunk id % 16).
   const uint16_t *hsrc[SJ];
-  int lds_off[SJ];
   bool hvalid[SJ];
 #pragma unroll
   for (int j = 0; j < SJ; ++j) {
-    const int id = tid + 256 * j;
-    const int row = id / CPR, c = id % CPR;
+    const int row = (tid >> 4) + 16 * j;
     hvalid[j] = row < P.num_rows;
     const int src = hvalid[j] ? (P.row_index ? P.row_index[row] : row) : 0;
-    hsrc[j] = P.hidden + static_cast<int64_t>(src) * P.hidden_stride + 8 * c;
-    lds_off[j] = row * kSmRow + 8 * c;
+    hsrc[j] = P.hidden + static_cast<int64_t>(src) * P.hidden_stride + 8 * (tid & 15);
   }
+  const int hoff = (tid >> 4) * kHRow + 8 * (tid & 15);
   sm_u32x4 st[SJ];
   auto stage_load = [&](int t) {
 #pragma unroll
@@ -102,52 +113,59 @@ __global__ __launch_bounds__(256) void lm_head_argmax_kernel(const LmHeadParams 
   };
   auto stage_store = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < SJ; ++j) *reinterpret_cast<sm_u32x4 *>(&tile[buf][lds_off[j]]) = st[j];
+    for (int j = 0; j < SJ; ++j) *reinterpret_cast<sm_u32x4 *>(&htile[buf][hoff + 16 * j * kHRow]) = st[j];
   };
-  auto load_a = [&](SmFrag (&a)[NF], int t) {
+  auto load_w = [&](sm_u32x4 (&w)[4], int t) {
 #pragma unroll
-    for (int i = 0; i < NF; ++i)
-      a[i].u = __builtin_nontemporal_load(reinterpret_cast<const sm_u32x4 *>(wp + t * KT + 32 * i));
+    for (int j = 0; j < 4; ++j)
+      w[j] = __builtin_nontemporal_load(reinterpret_cast<const sm_u32x4 *>(wsrc[j] + t * KT));
   };
 
   sm_v4f32 acc[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) acc[nb] = sm_v4f32{0.f, 0.f, 0.f, 0.f};
-  auto compute = [&](const SmFrag (&a)[NF], int buf) {
-    const uint16_t *base = &tile[buf][r16 * kSmRow + 8 * g];
+  // Regroup one embedding tile through the wave's LDS area, then multiply.
+  auto consume = [&](const sm_u32x4 (&w)[4], int buf) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<sm_u32x4 *>(wmine + (4 * j) * KT + 8 * lane) = w[j];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    SmFrag a[NF];
+#pragma unroll
+    for (int i = 0; i < NF; ++i)
+      a[i].u = *reinterpret_cast<const sm_u32x4 *>(wmine + r16 * KT + 8 * ((4 * i + g) ^ r16));
+    const uint16_t *base = &htile[buf][r16 * kHRow + 8 * g];
 #pragma unroll
     for (int i = 0; i < NF; ++i) {
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
         SmFrag b;
-        b.u = *reinterpret_cast<const sm_u32x4 *>(base + 16 * nb * kSmRow + 32 * i);
+        b.u = *reinterpret_cast<const sm_u32x4 *>(base + 16 * nb * kHRow + 32 * i);
         if constexpr (__is_same(T, F16))
           acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i].h, b.h, acc[nb], 0, 0, 0);
         else
           acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].b, b.b, acc[nb], 0, 0, 0);
       }
     }
+    __builtin_amdgcn_wave_barrier();                    // fragment reads stay ahead of the next tile's writes
   };
 
-  SmFrag a0[NF], a1[NF];
-  load_a(a0, 0);
+  sm_u32x4 w0[4], w1[4];
+  load_w(w0, 0);
+  if (n_tiles > 1) load_w(w1, 1);
   stage_load(0);
   stage_store(0);
   __syncthreads();
   for (int t = 0; t < n_tiles; t += 2) {
-    if (t + 1 < n_tiles) {
-      load_a(a1, t + 1);
-      stage_load(t + 1);
-    }
-    compute(a0, 0);
+    if (t + 1 < n_tiles) stage_load(t + 1);
+    consume(w0, 0);
+    if (t + 2 < n_tiles) load_w(w0, t + 2);
     if (t + 1 < n_tiles) stage_store(1);
     __syncthreads();
     if (t + 1 >= n_tiles) break;
-    if (t + 2 < n_tiles) {
-      load_a(a0, t + 2);
-      stage_load(t + 2);
-    }
-    compute(a1, 1);
+    if (t + 2 < n_tiles) stage_load(t + 2);
+    consume(w1, 1);
+    if (t + 3 < n_tiles) load_w(w1, t + 3);
     if (t + 2 < n_tiles) stage_store(0);
     __syncthreads();
   }
@@ -257,9 +275,9 @@ extern "C" int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_st
     const dim3 grid(n_wg), block(256);
 #define MUX_LM_LAUNCH(TT)                                                                   \
   do {                                                                                      \
-    if (nb == 1) hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 1, 256>), grid, block, 0, st, P); \
-    else if (nb == 2) hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 2, 256>), grid, block, 0, st, P); \
-    else hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 4, 128>), grid, block, 0, st, P);    \
+    if (nb == 1) hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 1>), grid, block, 0, st, P); \
+    else if (nb == 2) hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 2>), grid, block, 0, st, P); \
+    else hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 4>), grid, block, 0, st, P);         \
   } while (0)
     if (dtype == MUXA_DTYPE_F16) MUX_LM_LAUNCH(F16);
     else MUX_LM_LAUNCH(BF16);
