@@ -216,9 +216,14 @@ int32_t mux_silu_and_mul(void *out, int64_t out_row_stride, const void *x, int64
  * it is NULL.  embedding: [embedding_rows >= vocab_size, hidden_size], the
  * lm_head weight (models/llama.py:317-323); hidden_size a multiple of 256.
  * next_tokens: DEVICE int64 [num_rows].  workspace: DEVICE,
- * mux_greedy_sample_workspace_bytes(vocab_size) bytes, 16-byte aligned, no
- * initialisation needed; calls that share it must not overlap. */
+ * mux_greedy_sample_workspace_bytes(vocab_size) bytes, 16-byte aligned, its
+ * first 256 bytes (an arrival counter) zeroed once before the first use
+ * (mux_greedy_sample_workspace_init, or any zero fill); every call leaves them
+ * zeroed again.  Calls that share a workspace must
+ * not overlap.  Nothing is allocated and no memset is recorded, so a call can
+ * be captured into a HIP graph. */
 size_t mux_greedy_sample_workspace_bytes(int32_t vocab_size);
+int32_t mux_greedy_sample_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
 int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_states, int64_t hidden_row_stride,
                           const int32_t *row_index, int32_t num_rows, const void *embedding,
                           int64_t embedding_row_stride, int32_t embedding_rows, int32_t vocab_size,

@@ -3,17 +3,26 @@
 // 200-232).  Both are bound by HBM: every input element is read once and every
 // output element written once, in 16-byte pieces.
 //
-//   rms_norm      one wave per token row: the row stays in registers between the
-//                 sum of squares and the scaling, so x is read once; the wave sum
-//                 is a DPP reduction, no LDS and no barrier.
+//   rms_norm      one wave per token row at a time: the row stays in registers
+//                 between the sum of squares and the scaling, so x is read once
+//                 (with non-temporal loads: 19.5 instead of 26 us for 4096 rows
+//                 of 6656); the wave sum is a DPP reduction, no LDS, no barrier.
 //                 out = T(x * rsqrt(mean(x^2) + eps)) * w, the product in T.
 //   silu_and_mul  one thread per 8 outputs: out = T(a / (1 + exp(-a))) * b for
 //                 x = [a | b], the product in T.
+#include <algorithm>
+
 #include "mux_common.h"
 
 namespace mux {
 
 typedef uint32_t mo_u32x4 __attribute__((ext_vector_type(4)));
+
+#ifndef MUX_RMS_WAVES_PER_CU
+#define MUX_RMS_WAVES_PER_CU 8
+#endif
+constexpr int kRmsWavesPerCu = MUX_RMS_WAVES_PER_CU;
+
 
 template <typename T>
 __device__ __forceinline__ void unpack8(const mo_u32x4 v, float (&f)[8]) {
@@ -47,64 +56,86 @@ __device__ __forceinline__ mo_u32x4 pack8(const float (&f)[8]) {
 }
 
 // CPL = 16-byte chunks a lane keeps (a row has hidden / 8 chunks, lane l takes
-// chunks l, l + 64, ...).  CPL = 0: rows of any length, x read twice.
+// chunks l, l + 64, ...).  A wave walks rows wave, wave + W, wave + 2 W, ... (W
+// waves in the grid) with the next row's loads issued before the current row is
+// reduced and stored, so that across the chip reads and writes overlap instead
+// of coming as one burst of each.  CPL = 0: rows of any length, x read twice.
 template <typename T, int CPL>
 __global__ __launch_bounds__(256) void rms_norm_kernel(uint16_t *__restrict__ out, int64_t out_stride,
                                                        const uint16_t *__restrict__ x, int64_t x_stride,
                                                        const uint16_t *__restrict__ weight, float eps, int hidden,
                                                        int num_rows) {
   const int lane = threadIdx.x & 63;
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= num_rows) return;
+  const int first = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int step = gridDim.x * 4;
+  if (first >= num_rows) return;
   const int nchunks = hidden >> 3;
-  const mo_u32x4 *xr = reinterpret_cast<const mo_u32x4 *>(x + row * x_stride);
   const mo_u32x4 *wr = reinterpret_cast<const mo_u32x4 *>(weight);
-  mo_u32x4 *outr = reinterpret_cast<mo_u32x4 *>(out + row * out_stride);
-  float ss = 0.f;
+  const float inv_n = 1.0f / static_cast<float>(hidden);
   if constexpr (CPL > 0) {
-    mo_u32x4 v[CPL];
+    auto load_row = [&](mo_u32x4 (&v)[CPL], int row) {
+      const mo_u32x4 *xr = reinterpret_cast<const mo_u32x4 *>(x + row * x_stride);
 #pragma unroll
-    for (int i = 0; i < CPL; ++i) {
-      const int c = lane + 64 * i;
-      v[i] = c < nchunks ? xr[c] : mo_u32x4{0, 0, 0, 0};
-    }
+      for (int i = 0; i < CPL; ++i) {
+        const int c = lane + 64 * i;
+        v[i] = c < nchunks ? __builtin_nontemporal_load(&xr[c]) : mo_u32x4{0, 0, 0, 0};
+      }
+    };
+    auto finish_row = [&](const mo_u32x4 (&v)[CPL], int row) {
+      float ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < CPL; ++i) {
-      float f[8];
-      unpack8<T>(v[i], f);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(f[j], f[j], ss);
-    }
-    ss = wave_sum(ss);
-    const float s = rsqrtf(ss / static_cast<float>(hidden) + eps);
-#pragma unroll
-    for (int i = 0; i < CPL; ++i) {
-      const int c = lane + 64 * i;
-      if (c < nchunks) {
-        float f[8], w[8];
+      for (int i = 0; i < CPL; ++i) {
+        float f[8];
         unpack8<T>(v[i], f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(f[j], f[j], ss);
+      }
+      ss = wave_sum(ss);
+      const float s = rsqrtf(ss * inv_n + eps);
+      mo_u32x4 *outr = reinterpret_cast<mo_u32x4 *>(out + row * out_stride);
+#pragma unroll
+      for (int i = 0; i < CPL; ++i) {
+        const int c = lane + 64 * i;
+        if (c < nchunks) {
+          float f[8], w[8];
+          unpack8<T>(v[i], f);
+          unpack8<T>(wr[c], w);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) f[j] = round_to<T>(f[j] * s) * w[j];
+          outr[c] = pack8<T>(f);
+        }
+      }
+    };
+    mo_u32x4 a[CPL], b[CPL];
+    load_row(a, first);
+    for (int row = first; row < num_rows; row += 2 * step) {
+      if (row + step < num_rows) load_row(b, row + step);
+      finish_row(a, row);
+      if (row + step >= num_rows) break;
+      if (row + 2 * step < num_rows) load_row(a, row + 2 * step);
+      finish_row(b, row + step);
+    }
+  } else {
+    for (int row = first; row < num_rows; row += step) {
+      const mo_u32x4 *xr = reinterpret_cast<const mo_u32x4 *>(x + row * x_stride);
+      mo_u32x4 *outr = reinterpret_cast<mo_u32x4 *>(out + row * out_stride);
+      float ss = 0.f;
+      for (int c = lane; c < nchunks; c += 64) {
+        float f[8];
+        unpack8<T>(xr[c], f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(f[j], f[j], ss);
+      }
+      ss = wave_sum(ss);
+      const float s = rsqrtf(ss * inv_n + eps);
+      for (int c = lane; c < nchunks; c += 64) {
+        float f[8], w[8];
+        unpack8<T>(xr[c], f);
         unpack8<T>(wr[c], w);
 #pragma unroll
         for (int j = 0; j < 8; ++j) f[j] = round_to<T>(f[j] * s) * w[j];
         outr[c] = pack8<T>(f);
       }
-    }
-  } else {
-    for (int c = lane; c < nchunks; c += 64) {
-      float f[8];
-      unpack8<T>(xr[c], f);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(f[j], f[j], ss);
-    }
-    ss = wave_sum(ss);
-    const float s = rsqrtf(ss / static_cast<float>(hidden) + eps);
-    for (int c = lane; c < nchunks; c += 64) {
-      float f[8], w[8];
-      unpack8<T>(xr[c], f);
-      unpack8<T>(wr[c], w);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) f[j] = round_to<T>(f[j] * s) * w[j];
-      outr[c] = pack8<T>(f);
     }
   }
 }
@@ -118,7 +149,7 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(uint16_t *__restrict_
   const int64_t t = id / d8;
   const int c = static_cast<int>(id - t * d8);
   const mo_u32x4 *xr = reinterpret_cast<const mo_u32x4 *>(x + t * x_stride);
-  const mo_u32x4 av = xr[c], bv = xr[d8 + c];
+  const mo_u32x4 av = __builtin_nontemporal_load(&xr[c]), bv = __builtin_nontemporal_load(&xr[d8 + c]);
   float a[8], b[8];
   unpack8<T>(av, a);
   unpack8<T>(bv, b);
@@ -146,7 +177,16 @@ extern "C" int32_t mux_rms_norm(void *out, int64_t out_row_stride, const void *x
     return MUXA_EINVAL;
   if (num_tokens == 0) return MUXA_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 grid((num_tokens + 3) / 4), block(256);
+  // At most kRmsWavesPerCu waves per CU; rows beyond that are walked in sequence.
+  static const int cus = [] {                      // compute units of the current device, asked once
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      return v;
+    return 256;
+  }();
+  const int max_wgs = cus * kRmsWavesPerCu / 4;
+  const dim3 grid(std::min((num_tokens + 3) / 4, max_wgs)), block(256);
   uint16_t *o = static_cast<uint16_t *>(out);
   const uint16_t *xi = static_cast<const uint16_t *>(x), *w = static_cast<const uint16_t *>(weight);
   const int nchunks = hidden_size / 8;

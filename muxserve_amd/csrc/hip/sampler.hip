@@ -4,24 +4,29 @@
 // reads the [vocab, hidden] matrix once (262 MB for a 7B model) and a few rows of
 // hidden states, so the kernel is bound by HBM.
 //
-// lm_head_argmax_kernel<T, NB>: a workgroup owns 64 vocabulary rows (16 per
-// wave) and up to 16 NB sampled rows of hidden states, and walks the hidden
-// dimension in tiles of 128.
-//   * Hidden states: the tile [16 NB][128] is staged in LDS, shared by the four
-//     waves, double-buffered, one barrier per tile.
+// lm_head_argmax_kernel<T, NB, NW>: a workgroup of NW waves owns 16 NW
+// vocabulary rows (16 per wave) and up to 16 NB sampled rows of hidden states,
+// and walks the hidden dimension in tiles of 128.
+//   * Hidden states: the tile [16 NB][128] is staged in LDS, shared by the
+//     waves, double-buffered, one barrier per tile.  Every workgroup reads all
+//     of the sampled hidden states (from L2), so large vocabularies use 8 waves
+//     per workgroup: half as many workgroups, half that traffic.
 //   * Embedding rows: the MFMA A operand wants lane l to hold row l % 16
 //     (v_mfma_f32_16x16x32: columns 8 (l / 16) .. +7 of a 32-column slice) -
 //     loaded that way, every 16 lanes would touch 16 different rows with 16 bytes
 //     each.  Instead a load instruction takes 4 rows x 256 contiguous bytes
-//     (16 lanes per row), two tiles ahead of their use, and the wave regroups
+//     (16 lanes per row), two tiles ahead of their use (deeper makes no difference), and the wave regroups
 //     its 4 KiB tile through a private LDS area: 16-byte chunk c of row r sits at
 //     position c ^ r of the row, so both the row-wise writes and the
 //     column-wise fragment reads are free of bank conflicts.
 // Accumulators hold logits[vocab row 4 (l / 16) + i][sampled row l % 16]; each is
-// rounded to the storage type (the reference compares logits of that type),
-// reduced to the workgroup's (max, lowest index) per sampled row and written to
-// a partial table.  argmax_finish_kernel reduces the table: one wave per
-// sampled row.
+// rounded to the storage type (the reference compares logits of that type) and
+// reduced to the workgroup's (max, lowest index) per sampled row, which goes to
+// the workgroup's line of a table as a 64-bit key (ordered logit bits << 32 |
+// ~index).  The last workgroup to arrive (a counter tells it) takes the maximum
+// of every column of the table, writes the token ids and leaves the counter at
+// zero for the next launch.  (Atomic max on one key per sampled row instead of
+// the table serialises 16000 atomics on two cache lines: +30 us per launch.)
 #include "mux_common.h"
 
 namespace mux {
@@ -38,7 +43,10 @@ union SmFrag {
 };
 
 constexpr int kSmTile = 256;              // the hidden size must be a multiple of this
-constexpr int kSmVocabPerWg = 64;
+constexpr int kSmMaxRowsPerPass = 64;
+#ifndef MUX_SM_PREFETCH_TILES
+#define MUX_SM_PREFETCH_TILES 2
+#endif
 
 struct LmHeadParams {
   const uint16_t *hidden;
@@ -47,9 +55,16 @@ struct LmHeadParams {
   const uint16_t *weight;
   int64_t weight_stride;
   int32_t hidden_size, vocab, num_rows;
-  float *part_val;                        // [workgroups][16 NB]
-  int32_t *part_idx;
+  uint32_t *counter;                      // workgroups arrived, zero between launches
+  unsigned long long *table;              // [workgroups][16 NB] keys, written before they are read
+  int64_t *next_tokens;
 };
+
+// Float bits that compare like the floats as unsigned integers.
+__device__ __forceinline__ uint32_t ordered_bits(float f) {
+  const uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
 
 template <typename T>
 __device__ __forceinline__ float sm_round(float f) {
@@ -65,18 +80,20 @@ __device__ __forceinline__ void take_better(float &v, int &i, float ov, int oi) 
   }
 }
 
-template <typename T, int NB>
-__global__ __launch_bounds__(256) void lm_head_argmax_kernel(const LmHeadParams P) {
+template <typename T, int NB, int NW>
+__global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadParams P) {
   constexpr int KT = 128;                             // hidden elements per tile
   constexpr int ROWS = 16 * NB;                       // sampled rows held in LDS
   constexpr int CPR = KT / 8;                         // 16-byte chunks per tile row (16)
-  constexpr int SJ = ROWS * CPR / 256;                // hidden-state staging chunks per thread (= NB)
+  constexpr int RPP = 4 * NW;                         // hidden-state rows staged per pass of the workgroup
+  constexpr int SJ = (ROWS + RPP - 1) / RPP;          // staging chunks per thread
   constexpr int NF = KT / 32;                         // MFMA column slices per tile (4)
   constexpr int kHRow = KT + 8;     // LDS row pitch: 16 bytes of padding keep b128 reads off each other's banks
   __shared__ __attribute__((aligned(16))) uint16_t htile[2][ROWS * kHRow];
-  __shared__ __attribute__((aligned(16))) uint16_t wtile[4][16 * KT];      // one 4 KiB area per wave
-  __shared__ float red_v[4][ROWS];
-  __shared__ int red_i[4][ROWS];
+  __shared__ __attribute__((aligned(16))) uint16_t wtile[NW][16 * KT];     // one 4 KiB area per wave
+  __shared__ float red_v[NW][ROWS];
+  __shared__ int red_i[NW][ROWS];
+  __shared__ int s_last;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, g = lane >> 4;
   const int n_tiles = P.hidden_size / KT;
@@ -84,7 +101,7 @@ __global__ __launch_bounds__(256) void lm_head_argmax_kernel(const LmHeadParams 
   // Embedding rows of this wave (rows past the vocabulary re-read its last row
   // and are masked at the end).  Load instruction j: lane l takes row
   // 4 j + l / 16, and of that row the chunk (l % 16) ^ row.
-  const int vrow0 = blockIdx.x * kSmVocabPerWg + 16 * wave;
+  const int vrow0 = blockIdx.x * (16 * NW) + 16 * wave;
   const uint16_t *wsrc[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -94,13 +111,14 @@ __global__ __launch_bounds__(256) void lm_head_argmax_kernel(const LmHeadParams 
   }
   uint16_t *const wmine = &wtile[wave][0];
 
-  // Hidden-state staging: chunk id = tid + 256 j -> (row id / 16, 16-byte chunk id % 16).
+  // Hidden-state staging: thread -> (row tid / 16 + RPP j, 16-byte chunk tid % 16).
   const uint16_t *hsrc[SJ];
-  bool hvalid[SJ];
+  bool hvalid[SJ], hstore[SJ];
 #pragma unroll
   for (int j = 0; j < SJ; ++j) {
-    const int row = (tid >> 4) + 16 * j;
-    hvalid[j] = row < P.num_rows;
+    const int row = (tid >> 4) + RPP * j;
+    hstore[j] = row < ROWS;
+    hvalid[j] = row < P.num_rows && hstore[j];
     const int src = hvalid[j] ? (P.row_index ? P.row_index[row] : row) : 0;
     hsrc[j] = P.hidden + static_cast<int64_t>(src) * P.hidden_stride + 8 * (tid & 15);
   }
@@ -113,7 +131,8 @@ __global__ __launch_bounds__(256) void lm_head_argmax_kernel(const LmHeadParams 
   };
   auto stage_store = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < SJ; ++j) *reinterpret_cast<sm_u32x4 *>(&htile[buf][hoff + 16 * j * kHRow]) = st[j];
+    for (int j = 0; j < SJ; ++j)
+      if (hstore[j]) *reinterpret_cast<sm_u32x4 *>(&htile[buf][hoff + RPP * j * kHRow]) = st[j];
   };
   auto load_w = [&](sm_u32x4 (&w)[4], int t) {
 #pragma unroll
@@ -150,24 +169,29 @@ __global__ __launch_bounds__(256) void lm_head_argmax_kernel(const LmHeadParams 
     __builtin_amdgcn_wave_barrier();                    // fragment reads stay ahead of the next tile's writes
   };
 
-  sm_u32x4 w0[4], w1[4];
-  load_w(w0, 0);
-  if (n_tiles > 1) load_w(w1, 1);
+  // PD embedding tiles per wave are in flight (register sets used in rotation;
+  // the rotation is unrolled so that every set is addressed statically).
+  constexpr int PD = MUX_SM_PREFETCH_TILES;
+  static_assert(PD % 2 == 0, "the hidden-state buffers alternate with the tile parity");
+  sm_u32x4 w[PD][4];
+#pragma unroll
+  for (int s2 = 0; s2 < PD; ++s2)
+    if (s2 < n_tiles) load_w(w[s2], s2);
   stage_load(0);
   stage_store(0);
   __syncthreads();
-  for (int t = 0; t < n_tiles; t += 2) {
-    if (t + 1 < n_tiles) stage_load(t + 1);
-    consume(w0, 0);
-    if (t + 2 < n_tiles) load_w(w0, t + 2);
-    if (t + 1 < n_tiles) stage_store(1);
-    __syncthreads();
-    if (t + 1 >= n_tiles) break;
-    if (t + 2 < n_tiles) stage_load(t + 2);
-    consume(w1, 1);
-    if (t + 3 < n_tiles) load_w(w1, t + 3);
-    if (t + 2 < n_tiles) stage_store(0);
-    __syncthreads();
+  for (int t0 = 0; t0 < n_tiles; t0 += PD) {
+#pragma unroll
+    for (int s2 = 0; s2 < PD; ++s2) {
+      const int t = t0 + s2;
+      if (t < n_tiles) {
+        if (t + 1 < n_tiles) stage_load(t + 1);
+        consume(w[s2], s2 & 1);
+        if (t + PD < n_tiles) load_w(w[s2], t + PD);
+        if (t + 1 < n_tiles) stage_store((s2 + 1) & 1);
+        __syncthreads();
+      }
+    }
   }
 
   // Lane holds logits[vocab row vrow0 + 4 g + i][sampled row 16 nb + r16].
@@ -193,44 +217,89 @@ __global__ __launch_bounds__(256) void lm_head_argmax_kernel(const LmHeadParams 
     }
   }
   __syncthreads();
+  // The workgroup's result per sampled row goes to its line of the table as a
+  // 64-bit key (ordered logit bits << 32 | ~index: a larger key is a better
+  // logit or, between equal logits, a lower index).
   if (tid < ROWS) {
     float bv = red_v[0][tid];
     int bi = red_i[0][tid];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) take_better(bv, bi, red_v[w][tid], red_i[w][tid]);
-    P.part_val[static_cast<int64_t>(blockIdx.x) * ROWS + tid] = bv;
-    P.part_idx[static_cast<int64_t>(blockIdx.x) * ROWS + tid] = bi;
+    for (int w = 1; w < NW; ++w) take_better(bv, bi, red_v[w][tid], red_i[w][tid]);
+    const unsigned long long key = (static_cast<unsigned long long>(ordered_bits(bv)) << 32) |
+                                   (0xffffffffu - static_cast<uint32_t>(bi));
+    __hip_atomic_store(&P.table[static_cast<int64_t>(blockIdx.x) * ROWS + tid], key, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
   }
-}
-
-// One wave per sampled row: lanes stride over the workgroups' partial results.
-__global__ __launch_bounds__(64) void argmax_finish_kernel(int64_t *__restrict__ next_tokens,
-                                                           const float *__restrict__ part_val,
-                                                           const int32_t *__restrict__ part_idx, int n_parts,
-                                                           int rows_pitch) {
-  const int r = blockIdx.x, lane = threadIdx.x;
-  float bv = -__builtin_inff();
-  int bi = 0x7fffffff;
-  for (int b = lane; b < n_parts; b += 64)
-    take_better(bv, bi, part_val[static_cast<int64_t>(b) * rows_pitch + r],
-                part_idx[static_cast<int64_t>(b) * rows_pitch + r]);
+  // The table is written and read with device-coherent accesses (they bypass
+  // the per-XCD L2), so ordering them against the counter takes only a
+  // workgroup-scope fence, i.e. a wait.  A device-scope fence would write back
+  // and invalidate this XCD's L2, which holds the hidden states every other
+  // workgroup is still reading (measured: +30 us per launch).
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (tid == 0)
+    s_last = __hip_atomic_fetch_add(P.counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1;
+  __syncthreads();
+  if (!s_last) return;
+  // Last workgroup to arrive: thread -> (sampled row tid % ROWS, slice
+  // tid / ROWS of the workgroups), sixteen loads in flight.
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  constexpr int SLICES = 64 * NW / ROWS;
+  __shared__ unsigned long long fin[SLICES][ROWS];
+  const int row = tid % ROWS, slice = tid / ROWS;
+  unsigned long long best = 0;
+  const int n_wg = gridDim.x;
+  for (int b0 = slice; b0 < n_wg; b0 += 16 * SLICES) {
+    unsigned long long v[16];
 #pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const float ov = __shfl_xor(bv, off);
-    const int oi = __shfl_xor(bi, off);
-    take_better(bv, bi, ov, oi);
+    for (int j = 0; j < 16; ++j) {
+      const int b = b0 + j * SLICES;
+      v[j] = b < n_wg ? __hip_atomic_load(&P.table[static_cast<int64_t>(b) * ROWS + row], __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT)
+                      : 0ull;
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j) best = v[j] > best ? v[j] : best;
   }
-  if (lane == 0) next_tokens[r] = bi == 0x7fffffff ? 0 : bi;   // every logit NaN: token 0
+  fin[slice][row] = best;
+  __syncthreads();
+  if (tid < P.num_rows) {
+    unsigned long long k = fin[0][tid];
+#pragma unroll
+    for (int sl = 1; sl < SLICES; ++sl) k = fin[sl][tid] > k ? fin[sl][tid] : k;
+    const uint32_t idx = 0xffffffffu - static_cast<uint32_t>(k);
+    P.next_tokens[tid] = idx < static_cast<uint32_t>(P.vocab) ? idx : 0;   // every logit NaN: token 0
+  }
+  if (tid == 0) __hip_atomic_store(P.counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-constexpr int kSmMaxRowsPerPass = 64;
+__global__ void sampler_zero_kernel(uint32_t *p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+constexpr size_t kSmCounterBytes = 256;        // the arrival counter, then the table
+#ifndef MUX_SM_EIGHT_WAVE_MIN_WGS
+#define MUX_SM_EIGHT_WAVE_MIN_WGS 192
+#endif
+constexpr int kSmEightWaveMinWgs = MUX_SM_EIGHT_WAVE_MIN_WGS;
 
 }  // namespace mux
 
 extern "C" size_t mux_greedy_sample_workspace_bytes(int32_t vocab_size) {
   if (vocab_size <= 0) return 0;
-  const size_t n_wg = (static_cast<size_t>(vocab_size) + mux::kSmVocabPerWg - 1) / mux::kSmVocabPerWg;
-  return n_wg * mux::kSmMaxRowsPerPass * (sizeof(float) + sizeof(int32_t));
+  const size_t n_wg = (static_cast<size_t>(vocab_size) + 63) / 64;            // the most workgroups a launch uses
+  return mux::kSmCounterBytes + n_wg * mux::kSmMaxRowsPerPass * sizeof(unsigned long long);
+}
+
+extern "C" int32_t mux_greedy_sample_workspace_init(void *workspace, size_t workspace_bytes, void *stream) {
+  using namespace mux;
+  if (!workspace || workspace_bytes < kSmCounterBytes || (reinterpret_cast<uintptr_t>(workspace) & 15u))
+    return MUXA_EWORKSPACE;
+  hipLaunchKernelGGL(sampler_zero_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<uint32_t *>(workspace), static_cast<int>(kSmCounterBytes / 4));
+  MUX_HIP_TRY(hipGetLastError());
+  return MUXA_OK;
 }
 
 extern "C" int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_states, int64_t hidden_row_stride,
@@ -253,11 +322,11 @@ extern "C" int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_st
       (reinterpret_cast<uintptr_t>(workspace) & 15u))
     return MUXA_EWORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const int n_wg = (vocab_size + kSmVocabPerWg - 1) / kSmVocabPerWg;
-  float *part_val = static_cast<float *>(workspace);
-  int32_t *part_idx = reinterpret_cast<int32_t *>(part_val + static_cast<size_t>(n_wg) * kSmMaxRowsPerPass);
+  // 8 waves (128 vocabulary rows) per workgroup once that still gives the chip enough workgroups.
+  const int nw = (vocab_size + 127) / 128 >= kSmEightWaveMinWgs ? 8 : 4;
+  const int n_wg = (vocab_size + 16 * nw - 1) / (16 * nw);
   // At most 64 sampled rows per pass over the matrix; larger batches take
-  // several passes that reuse the partial table one after the other.
+  // several passes, one after the other on the stream.
   for (int r0 = 0; r0 < num_rows; r0 += kSmMaxRowsPerPass) {
     const int rows = min(num_rows - r0, kSmMaxRowsPerPass);
     LmHeadParams P;
@@ -269,21 +338,26 @@ extern "C" int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_st
     P.hidden_size = hidden_size;
     P.vocab = vocab_size;
     P.num_rows = rows;
-    P.part_val = part_val;
-    P.part_idx = part_idx;
+    P.counter = static_cast<uint32_t *>(workspace);
+    P.table = reinterpret_cast<unsigned long long *>(static_cast<char *>(workspace) + kSmCounterBytes);
+    P.next_tokens = next_tokens + r0;
     const int nb = rows <= 16 ? 1 : (rows <= 32 ? 2 : 4);
-    const dim3 grid(n_wg), block(256);
-#define MUX_LM_LAUNCH(TT)                                                                   \
-  do {                                                                                      \
-    if (nb == 1) hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 1>), grid, block, 0, st, P); \
-    else if (nb == 2) hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 2>), grid, block, 0, st, P); \
-    else hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 4>), grid, block, 0, st, P);         \
+    const dim3 grid(n_wg), block(64 * nw);
+#define MUX_LM_LAUNCH_NW(TT, NWV)                                                                    \
+  do {                                                                                               \
+    if (nb == 1) hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 1, NWV>), grid, block, 0, st, P);      \
+    else if (nb == 2) hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 2, NWV>), grid, block, 0, st, P); \
+    else hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 4, NWV>), grid, block, 0, st, P);              \
+  } while (0)
+#define MUX_LM_LAUNCH(TT)            \
+  do {                               \
+    if (nw == 8) MUX_LM_LAUNCH_NW(TT, 8); \
+    else MUX_LM_LAUNCH_NW(TT, 4);    \
   } while (0)
     if (dtype == MUXA_DTYPE_F16) MUX_LM_LAUNCH(F16);
     else MUX_LM_LAUNCH(BF16);
 #undef MUX_LM_LAUNCH
-    hipLaunchKernelGGL(argmax_finish_kernel, dim3(rows), dim3(64), 0, st, next_tokens + r0, part_val, part_idx, n_wg,
-                       16 * nb);
+#undef MUX_LM_LAUNCH_NW
   }
   MUX_HIP_TRY(hipGetLastError());
   return MUXA_OK;

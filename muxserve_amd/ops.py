@@ -290,7 +290,9 @@ def greedy_sample(embedding: torch.Tensor, hidden_states: torch.Tensor, vocab_si
                   row_index: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                   workspace: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
     """int64 [num_rows] on the device: argmax over v < vocab_size of
-    hidden_states[row] . embedding[v], row = row_index[r] (int32, device) or r."""
+    hidden_states[row] . embedding[v], row = row_index[r] (int32, device) or r.
+    A caller's own workspace must be zeroed once before its first use; every
+    call leaves it zeroed."""
     _need_cuda(embedding, hidden_states)
     if embedding.dim() != 2 or hidden_states.dim() != 2 or embedding.shape[1] != hidden_states.shape[1]:
         raise ValueError("embedding [V, hidden] and hidden_states [T, hidden] expected")
@@ -316,7 +318,7 @@ def greedy_sample(embedding: torch.Tensor, hidden_states: torch.Tensor, vocab_si
         key = (hidden_states.device, torch.cuda.current_stream(hidden_states.device).cuda_stream)
         workspace = _sample_workspaces.get(key)
         if workspace is None or workspace.numel() < need:
-            workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=hidden_states.device)
+            workspace = torch.zeros(max(need, 1), dtype=torch.uint8, device=hidden_states.device)   # born zeroed
             _sample_workspaces[key] = workspace
     rc = lib.mux_greedy_sample(out.data_ptr(), hidden_states.data_ptr(), _rows(hidden_states, "hidden_states"), ri_ptr,
                                num_rows, embedding.data_ptr(), _rows(embedding, "embedding"), embedding.shape[0],

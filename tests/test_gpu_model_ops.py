@@ -187,6 +187,24 @@ def test_greedy_sampler_module_prompt_and_decode_steps():
     _check_tokens(toks, emb, hid[:13], V, torch.float16, "decode step")
 
 
+def test_greedy_sample_leaves_its_counter_zeroed_and_the_workspace_reusable():
+    """One caller-owned workspace serves calls of different vocabulary sizes,
+    batch sizes and workgroup shapes one after the other."""
+    print("[case] greedy_sample workspace reuse", flush=True)
+    from muxserve_amd import _lib
+    g = torch.Generator().manual_seed(21)
+    ws = torch.full((_lib.attn().mux_greedy_sample_workspace_bytes(32000),), 0xAB, dtype=torch.uint8, device=DEV)
+    rc = _lib.attn().mux_greedy_sample_workspace_init(ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    for V, Hd, R in ((32000, 256, 3), (700, 512, 40), (24593, 256, 64), (32000, 256, 20), (129, 256, 1)):
+        emb = (torch.randn((V + 7, Hd), generator=g) * 0.1).half()
+        hid = torch.randn((R, Hd), generator=g).half()
+        toks = ops.greedy_sample(emb.to(DEV), hid.to(DEV), V, R, workspace=ws)
+        torch.cuda.synchronize()
+        _check_tokens(toks.cpu().tolist(), emb, hid, V, torch.float16, f"V={V} R={R}")
+        assert int(ws[:256].count_nonzero()) == 0, "arrival counter not left at zero"
+
+
 def test_model_ops_reject_malformed_arguments():
     x = torch.zeros((4, 4100), dtype=torch.float16, device=DEV)
     with pytest.raises(RuntimeError):
