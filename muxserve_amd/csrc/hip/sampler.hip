@@ -15,7 +15,7 @@
 //     (v_mfma_f32_16x16x32: columns 8 (l / 16) .. +7 of a 32-column slice) -
 //     loaded that way, every 16 lanes would touch 16 different rows with 16 bytes
 //     each.  Instead a load instruction takes 4 rows x 256 contiguous bytes
-//     (16 lanes per row), two tiles ahead of their use (deeper makes no difference), and the wave regroups
+//     (16 lanes per row), a tile ahead of their use (deeper makes no difference), and the wave regroups
 //     its 4 KiB tile through a private LDS area: 16-byte chunk c of row r sits at
 //     position c ^ r of the row, so both the row-wise writes and the
 //     column-wise fragment reads are free of bank conflicts.
@@ -97,6 +97,15 @@ __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadPar
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, g = lane >> 4;
   const int n_tiles = P.hidden_size / KT;
+  // Workgroups start their walk over the hidden dimension at different tiles
+  // (a dot product does not care about the order): with a row pitch that is a
+  // power of two - 8 KiB at hidden size 4096 - workgroups walking in step would
+  // all be reading the same few memory channels at any moment.
+  const int t_start = blockIdx.x % n_tiles;
+  auto tile_of = [&](int t) {
+    const int x = t + t_start;
+    return x >= n_tiles ? x - n_tiles : x;
+  };
 
   // Embedding rows of this wave (rows past the vocabulary re-read its last row
   // and are masked at the end).  Load instruction j: lane l takes row
@@ -123,13 +132,12 @@ __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadPar
     hsrc[j] = P.hidden + static_cast<int64_t>(src) * P.hidden_stride + 8 * (tid & 15);
   }
   const int hoff = (tid >> 4) * kHRow + 8 * (tid & 15);
-  sm_u32x4 st[SJ];
-  auto stage_load = [&](int t) {
+  auto stage_load = [&](sm_u32x4 (&st)[SJ], int t) {
 #pragma unroll
     for (int j = 0; j < SJ; ++j)
-      st[j] = hvalid[j] ? *reinterpret_cast<const sm_u32x4 *>(hsrc[j] + t * KT) : sm_u32x4{0, 0, 0, 0};
+      st[j] = hvalid[j] ? *reinterpret_cast<const sm_u32x4 *>(hsrc[j] + tile_of(t) * KT) : sm_u32x4{0, 0, 0, 0};
   };
-  auto stage_store = [&](int buf) {
+  auto stage_store = [&](const sm_u32x4 (&st)[SJ], int buf) {
 #pragma unroll
     for (int j = 0; j < SJ; ++j)
       if (hstore[j]) *reinterpret_cast<sm_u32x4 *>(&htile[buf][hoff + RPP * j * kHRow]) = st[j];
@@ -137,7 +145,7 @@ __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadPar
   auto load_w = [&](sm_u32x4 (&w)[4], int t) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      w[j] = __builtin_nontemporal_load(reinterpret_cast<const sm_u32x4 *>(wsrc[j] + t * KT));
+      w[j] = __builtin_nontemporal_load(reinterpret_cast<const sm_u32x4 *>(wsrc[j] + tile_of(t) * KT));
   };
 
   sm_v4f32 acc[NB];
@@ -169,26 +177,32 @@ __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadPar
     __builtin_amdgcn_wave_barrier();                    // fragment reads stay ahead of the next tile's writes
   };
 
-  // PD embedding tiles per wave are in flight (register sets used in rotation;
-  // the rotation is unrolled so that every set is addressed statically).
+  // PD tiles per wave are in flight: register sets used in rotation (unrolled,
+  // so every set is addressed statically).  Loads return in order, so the
+  // hidden-state part of a tile is requested together with - and just before -
+  // its embedding part: waiting for one never waits for a younger tile.
   constexpr int PD = MUX_SM_PREFETCH_TILES;
   static_assert(PD % 2 == 0, "the hidden-state buffers alternate with the tile parity");
-  sm_u32x4 w[PD][4];
+  sm_u32x4 w[PD][4], st[PD][SJ];
 #pragma unroll
   for (int s2 = 0; s2 < PD; ++s2)
-    if (s2 < n_tiles) load_w(w[s2], s2);
-  stage_load(0);
-  stage_store(0);
+    if (s2 < n_tiles) {
+      stage_load(st[s2], s2);
+      load_w(w[s2], s2);
+    }
+  stage_store(st[0], 0);
   __syncthreads();
   for (int t0 = 0; t0 < n_tiles; t0 += PD) {
 #pragma unroll
     for (int s2 = 0; s2 < PD; ++s2) {
       const int t = t0 + s2;
       if (t < n_tiles) {
-        if (t + 1 < n_tiles) stage_load(t + 1);
         consume(w[s2], s2 & 1);
-        if (t + PD < n_tiles) load_w(w[s2], t + PD);
-        if (t + 1 < n_tiles) stage_store((s2 + 1) & 1);
+        if (t + 1 < n_tiles) stage_store(st[(s2 + 1) % PD], (s2 + 1) & 1);
+        if (t + PD < n_tiles) {
+          stage_load(st[s2], t + PD);
+          load_w(w[s2], t + PD);
+        }
         __syncthreads();
       }
     }
