@@ -804,14 +804,19 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
   // Block ids of the step at tb: x, y for the K tokens tb + h and tb + 16 + h,
   // z for the V tokens tb + 8 g .. +7 (0 past t1).  Clamped so that a corrupt
   // table entry reads the wrong block instead of faulting the GPU.
+  // Raw table entries; they are clamped where they are used, so that nothing
+  // waits for them at the point of the load.
   auto load_ids = [&](int tb) {
     int3 id = make_int3(0, 0, 0);
-    if (tb + h < t1) id.x = min(max(trow[(tb + h) / BS], 0), last_block);
-    if (tb + 16 + h < t1) id.y = min(max(trow[(tb + 16 + h) / BS], 0), last_block);
-    if (tb + 8 * g < t1) id.z = min(max(trow[(tb + 8 * g) / BS], 0), last_block);
+    if (tb + h < t1) id.x = trow[(tb + h) / BS];
+    if (tb + 16 + h < t1) id.y = trow[(tb + 16 + h) / BS];
+    if (tb + 8 * g < t1) id.z = trow[(tb + 8 * g) / BS];
     return id;
   };
   auto issue = [&](GqaTile &r, int tb, int3 id) {
+    id.x = min(max(id.x, 0), last_block);
+    id.y = min(max(id.y, 0), last_block);
+    id.z = min(max(id.z, 0), last_block);
 #pragma unroll
     for (int tg = 0; tg < 2; ++tg) {
       const int tok = tb + 16 * tg + h;
@@ -910,26 +915,31 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
   };
 
   // Two register sets: the loads of the next step are in flight while the
-  // current one is consumed, and the block ids run one step further ahead.
+  // current one is consumed.  Vector loads return in order, so waiting for a
+  // step's block ids also waits for every load issued before them: the ids of
+  // step s + 2 are therefore requested BEFORE the K/V loads of step s + 1 go
+  // out (two id registers in rotation), and waiting for them never waits for
+  // K/V that is still wanted in flight.
   int tb = u.t0 + kGqaTile * wave;
   if (tb < t1) {
     GqaTile ra, rb;
-    issue(ra, tb, load_ids(tb));
-    int3 ids_next = make_int3(0, 0, 0);
-    if (tb + kStep < t1) ids_next = load_ids(tb + kStep);
+    int3 ids_a = load_ids(tb);
+    int3 ids_b = make_int3(0, 0, 0);
+    if (tb + kStep < t1) ids_b = load_ids(tb + kStep);
+    issue(ra, tb, ids_a);
     while (true) {
       const bool has_b = tb + kStep < t1;
       if (has_b) {
-        issue(rb, tb + kStep, ids_next);
-        if (tb + 2 * kStep < t1) ids_next = load_ids(tb + 2 * kStep);
+        if (tb + 2 * kStep < t1) ids_a = load_ids(tb + 2 * kStep);
+        issue(rb, tb + kStep, ids_b);
       }
       compute(ra, tb);
       if (!has_b) break;
       tb += kStep;
       const bool has_a = tb + kStep < t1;
       if (has_a) {
-        issue(ra, tb + kStep, ids_next);
-        if (tb + 2 * kStep < t1) ids_next = load_ids(tb + 2 * kStep);
+        if (tb + 2 * kStep < t1) ids_b = load_ids(tb + 2 * kStep);
+        issue(ra, tb + kStep, ids_a);
       }
       compute(rb, tb);
       if (!has_a) break;
