@@ -4,8 +4,8 @@
 // reads the [vocab, hidden] matrix once (262 MB for a 7B model) and a few rows of
 // hidden states, so the kernel is bound by HBM.
 //
-// lm_head_argmax_kernel<T, NB, NW>: a workgroup of NW waves owns 16 NW
-// vocabulary rows (16 per wave) and up to 16 NB sampled rows of hidden states,
+// lm_head_argmax_kernel<T, NB, NW, RB>: a workgroup of NW waves owns 16 NW RB
+// vocabulary rows (RB blocks of 16 per wave) and up to 16 NB sampled rows of hidden states,
 // and walks the hidden dimension in tiles of 128.
 //   * Hidden states: the tile [16 NB][128] is staged in LDS, shared by the
 //     waves, double-buffered, one barrier per tile.  Every workgroup reads all
@@ -80,7 +80,7 @@ __device__ __forceinline__ void take_better(float &v, int &i, float ov, int oi) 
   }
 }
 
-template <typename T, int NB, int NW>
+template <typename T, int NB, int NW, int RB>
 __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadParams P) {
   constexpr int KT = 128;                             // hidden elements per tile
   constexpr int ROWS = 16 * NB;                       // sampled rows held in LDS
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadPar
   constexpr int NF = KT / 32;                         // MFMA column slices per tile (4)
   constexpr int kHRow = KT + 8;     // LDS row pitch: 16 bytes of padding keep b128 reads off each other's banks
   __shared__ __attribute__((aligned(16))) uint16_t htile[2][ROWS * kHRow];
-  __shared__ __attribute__((aligned(16))) uint16_t wtile[NW][16 * KT];     // one 4 KiB area per wave
+  __shared__ __attribute__((aligned(16))) uint16_t wtile[NW][RB][16 * KT];  // 4 KiB per wave and row block
   __shared__ float red_v[NW][ROWS];
   __shared__ int red_i[NW][ROWS];
   __shared__ int s_last;
@@ -110,15 +110,17 @@ __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadPar
   // Embedding rows of this wave (rows past the vocabulary re-read its last row
   // and are masked at the end).  Load instruction j: lane l takes row
   // 4 j + l / 16, and of that row the chunk (l % 16) ^ row.
-  const int vrow0 = blockIdx.x * (16 * NW) + 16 * wave;
-  const uint16_t *wsrc[4];
+  const int vrow0 = blockIdx.x * (16 * NW * RB) + 16 * RB * wave;
+  const uint16_t *wsrc[RB][4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int row = 4 * j + g;
-    const int lrow = min(vrow0 + row, P.vocab - 1);
-    wsrc[j] = P.weight + static_cast<int64_t>(lrow) * P.weight_stride + 8 * (r16 ^ row);
-  }
-  uint16_t *const wmine = &wtile[wave][0];
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = 4 * j + g;
+      const int lrow = min(vrow0 + 16 * rb + row, P.vocab - 1);
+      wsrc[rb][j] = P.weight + static_cast<int64_t>(lrow) * P.weight_stride + 8 * (r16 ^ row);
+    }
+  uint16_t *const wmine = &wtile[wave][0][0];
 
   // Hidden-state staging: thread -> (row tid / 16 + RPP j, 16-byte chunk tid % 16).
   const uint16_t *hsrc[SJ];
@@ -142,25 +144,35 @@ __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadPar
     for (int j = 0; j < SJ; ++j)
       if (hstore[j]) *reinterpret_cast<sm_u32x4 *>(&htile[buf][hoff + RPP * j * kHRow]) = st[j];
   };
-  auto load_w = [&](sm_u32x4 (&w)[4], int t) {
+  auto load_w = [&](sm_u32x4 (&w)[RB][4], int t) {
+    const int off = tile_of(t) * KT;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      w[j] = __builtin_nontemporal_load(reinterpret_cast<const sm_u32x4 *>(wsrc[j] + tile_of(t) * KT));
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        w[rb][j] = __builtin_nontemporal_load(reinterpret_cast<const sm_u32x4 *>(wsrc[rb][j] + off));
   };
 
-  sm_v4f32 acc[NB];
+  sm_v4f32 acc[RB][NB];
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) acc[nb] = sm_v4f32{0.f, 0.f, 0.f, 0.f};
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[rb][nb] = sm_v4f32{0.f, 0.f, 0.f, 0.f};
   // Regroup one embedding tile through the wave's LDS area, then multiply.
-  auto consume = [&](const sm_u32x4 (&w)[4], int buf) {
+  auto consume = [&](const sm_u32x4 (&w)[RB][4], int buf) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) *reinterpret_cast<sm_u32x4 *>(wmine + (4 * j) * KT + 8 * lane) = w[j];
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        *reinterpret_cast<sm_u32x4 *>(wmine + rb * 16 * KT + (4 * j) * KT + 8 * lane) = w[rb][j];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    SmFrag a[NF];
+    SmFrag a[RB][NF];
 #pragma unroll
-    for (int i = 0; i < NF; ++i)
-      a[i].u = *reinterpret_cast<const sm_u32x4 *>(wmine + r16 * KT + 8 * ((4 * i + g) ^ r16));
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int i = 0; i < NF; ++i)
+        a[rb][i].u = *reinterpret_cast<const sm_u32x4 *>(wmine + rb * 16 * KT + r16 * KT + 8 * ((4 * i + g) ^ r16));
     const uint16_t *base = &htile[buf][r16 * kHRow + 8 * g];
 #pragma unroll
     for (int i = 0; i < NF; ++i) {
@@ -168,10 +180,13 @@ __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadPar
       for (int nb = 0; nb < NB; ++nb) {
         SmFrag b;
         b.u = *reinterpret_cast<const sm_u32x4 *>(base + 16 * nb * kHRow + 32 * i);
-        if constexpr (__is_same(T, F16))
-          acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i].h, b.h, acc[nb], 0, 0, 0);
-        else
-          acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].b, b.b, acc[nb], 0, 0, 0);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {      // one hidden-state fragment serves every row block of the wave
+          if constexpr (__is_same(T, F16))
+            acc[rb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[rb][i].h, b.h, acc[rb][nb], 0, 0, 0);
+          else
+            acc[rb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rb][i].b, b.b, acc[rb][nb], 0, 0, 0);
+        }
       }
     }
     __builtin_amdgcn_wave_barrier();                    // fragment reads stay ahead of the next tile's writes
@@ -183,7 +198,7 @@ __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadPar
   // its embedding part: waiting for one never waits for a younger tile.
   constexpr int PD = MUX_SM_PREFETCH_TILES;
   static_assert(PD % 2 == 0, "the hidden-state buffers alternate with the tile parity");
-  sm_u32x4 w[PD][4], st[PD][SJ];
+  sm_u32x4 w[PD][RB][4], st[PD][SJ];
 #pragma unroll
   for (int s2 = 0; s2 < PD; ++s2)
     if (s2 < n_tiles) {
@@ -208,17 +223,19 @@ __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadPar
     }
   }
 
-  // Lane holds logits[vocab row vrow0 + 4 g + i][sampled row 16 nb + r16].
+  // Lane holds logits[vocab row vrow0 + 16 rb + 4 g + i][sampled row 16 nb + r16].
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     float bv = -__builtin_inff();
     int bi = 0x7fffffff;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int vr = vrow0 + 4 * g + i;
-      const float val = sm_round<T>(acc[nb][i]);
-      if (vr < P.vocab) take_better(bv, bi, val, vr);
-    }
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int vr = vrow0 + 16 * rb + 4 * g + i;
+        const float val = sm_round<T>(acc[rb][nb][i]);
+        if (vr < P.vocab) take_better(bv, bi, val, vr);
+      }
 #pragma unroll
     for (int off = 16; off <= 32; off <<= 1) {
       const float ov = __shfl_xor(bv, off);
@@ -336,9 +353,13 @@ extern "C" int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_st
       (reinterpret_cast<uintptr_t>(workspace) & 15u))
     return MUXA_EWORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  // 8 waves (128 vocabulary rows) per workgroup once that still gives the chip enough workgroups.
-  const int nw = (vocab_size + 127) / 128 >= kSmEightWaveMinWgs ? 8 : 4;
-  const int n_wg = (vocab_size + 16 * nw - 1) / (16 * nw);
+  // 128 vocabulary rows per workgroup (8 waves) once that still gives the chip
+  // enough workgroups, else 64.  (Two row blocks per wave, RB = 2, halve the
+  // hidden-state fragment reads but measured slower with 4 waves per workgroup:
+  // 61 against 56 us at 64 sampled rows, hidden size 4096.)
+  const bool wide = (vocab_size + 127) / 128 >= kSmEightWaveMinWgs;
+  const int rows_per_wg = wide ? 128 : 64;
+  const int n_wg = (vocab_size + rows_per_wg - 1) / rows_per_wg;
   // At most 64 sampled rows per pass over the matrix; larger batches take
   // several passes, one after the other on the stream.
   for (int r0 = 0; r0 < num_rows; r0 += kSmMaxRowsPerPass) {
@@ -356,22 +377,23 @@ extern "C" int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_st
     P.table = reinterpret_cast<unsigned long long *>(static_cast<char *>(workspace) + kSmCounterBytes);
     P.next_tokens = next_tokens + r0;
     const int nb = rows <= 16 ? 1 : (rows <= 32 ? 2 : 4);
-    const dim3 grid(n_wg), block(64 * nw);
-#define MUX_LM_LAUNCH_NW(TT, NWV)                                                                    \
-  do {                                                                                               \
-    if (nb == 1) hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 1, NWV>), grid, block, 0, st, P);      \
-    else if (nb == 2) hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 2, NWV>), grid, block, 0, st, P); \
-    else hipLaunchKernelGGL((lm_head_argmax_kernel<TT, 4, NWV>), grid, block, 0, st, P);              \
-  } while (0)
-#define MUX_LM_LAUNCH(TT)            \
-  do {                               \
-    if (nw == 8) MUX_LM_LAUNCH_NW(TT, 8); \
-    else MUX_LM_LAUNCH_NW(TT, 4);    \
+    const dim3 grid(n_wg);
+#define MUX_LM_GO(TT, NBV, NWV, RBV) \
+  hipLaunchKernelGGL((lm_head_argmax_kernel<TT, NBV, NWV, RBV>), grid, dim3(64 * NWV), 0, st, P)
+#define MUX_LM_LAUNCH(TT)                  \
+  do {                                     \
+    if (!wide) {                           \
+      if (nb == 1) MUX_LM_GO(TT, 1, 4, 1); \
+      else if (nb == 2) MUX_LM_GO(TT, 2, 4, 1); \
+      else MUX_LM_GO(TT, 4, 4, 1);         \
+    } else if (nb == 1) MUX_LM_GO(TT, 1, 8, 1); \
+    else if (nb == 2) MUX_LM_GO(TT, 2, 8, 1);   \
+    else MUX_LM_GO(TT, 4, 8, 1);           \
   } while (0)
     if (dtype == MUXA_DTYPE_F16) MUX_LM_LAUNCH(F16);
     else MUX_LM_LAUNCH(BF16);
 #undef MUX_LM_LAUNCH
-#undef MUX_LM_LAUNCH_NW
+#undef MUX_LM_GO
   }
   MUX_HIP_TRY(hipGetLastError());
   return MUXA_OK;
