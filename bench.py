@@ -52,6 +52,8 @@ def parse():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-hint", action="store_true", help="do not pass the host-side sum of context lengths")
+    ap.add_argument("--no-prompt-order", action="store_true",
+                    help="prefill3: start the prompts' workgroups as packed instead of longest first")
     ap.add_argument("--unfused", action="store_true", help="one launch per model instead of one fused launch")
     ap.add_argument("--workload", default="mixed3_decode",
                     choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long", "model_ops"],
@@ -148,17 +150,19 @@ def bench_prefill3(args):
         cu = torch.from_numpy(m.cu_seqlens()).to(dev)
         slots, used = workloads.prefill_slot_mapping(m.prompt_lens, Hkv, bs, ids[cur:])
         cur += used
-        work.append((m, q, k, v, out, cu, torch.from_numpy(slots).to(dev), T))
+        order = torch.from_numpy(np.argsort(-m.prompt_lens, kind="stable").astype(np.int32)).to(dev)
+        work.append((m, q, k, v, out, cu, torch.from_numpy(slots).to(dev), T, order))
         flops += workloads.prefill_flops(m.prompt_lens, Hq)
         wbytes += workloads.cache_write_bytes(T, Hkv)
         tokens += T
 
     def attn(_):
-        for m, q, k, v, out, cu, slots, T in work:
-            ops.prefill_causal(out, q, k, v, cu, int(m.prompt_lens.max()), m.scale, m.num_kv_heads)
+        for m, q, k, v, out, cu, slots, T, order in work:
+            ops.prefill_causal(out, q, k, v, cu, int(m.prompt_lens.max()), m.scale, m.num_kv_heads,
+                               prompt_order=None if args.no_prompt_order else order)
 
     def write(_):
-        for m, q, k, v, out, cu, slots, T in work:
+        for m, q, k, v, out, cu, slots, T, order in work:
             ops.reshape_and_cache(k, v, k_pool, v_pool, slots, num_tokens=T)
 
     ms_a = _time(attn, args.steps, args.warmup)

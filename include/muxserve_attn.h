@@ -152,13 +152,17 @@ int32_t mux_paged_decode(void *out, int64_t out_row_stride, const void *q, int64
  *     out[t,hq,:] = softmax(scale * q[t,hq,:] . k[<=t,hk,:]) . v[<=t,hk,:]
  * on the fresh q,k,v (the pool is not read).  cu_seqlens: DEVICE int32
  * [num_prompts+1] prefix sums of InputMetadata.prompt_lens; max_prompt_len is
- * a host-side upper bound that sizes the grid. */
+ * a host-side upper bound that sizes the grid.  prompt_order: optional DEVICE
+ * int32 [num_prompts], a permutation of the prompts - the order in which their
+ * workgroups are started (the caller knows the lengths on the host; longest
+ * first keeps the longest prompt off the end of the launch); NULL: as packed.
+ * Results do not depend on it. */
 int32_t mux_prefill_causal(void *out, int64_t out_row_stride,
                            const void *q, int64_t q_row_stride,
                            const void *k, const void *v, int64_t kv_row_stride,
-                           const int32_t *cu_seqlens, int32_t num_prompts, int32_t max_prompt_len,
-                           int32_t num_q_heads, int32_t num_kv_heads, int32_t head_size,
-                           float scale, int32_t dtype, void *stream);
+                           const int32_t *cu_seqlens, const int32_t *prompt_order, int32_t num_prompts,
+                           int32_t max_prompt_len, int32_t num_q_heads, int32_t num_kv_heads,
+                           int32_t head_size, float scale, int32_t dtype, void *stream);
 
 /* ---- Rotary position embedding --------------------------------------------
  * The attention layer of the reference is PagedAttentionWithRoPE constructed

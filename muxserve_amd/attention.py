@@ -45,6 +45,7 @@ class InputMetadata:
     total_context_len: int = 0
     is_muxserve: bool = True                   # read at models/llama.py:285
     _cu_seqlens: Optional[torch.Tensor] = field(default=None, repr=False)
+    _prompt_order: Optional[torch.Tensor] = field(default=None, repr=False)
 
     def __post_init__(self):
         self.prompt_lens = [int(x) for x in self.prompt_lens]
@@ -65,6 +66,14 @@ class InputMetadata:
                 cu.append(cu[-1] + n)
             self._cu_seqlens = torch.tensor(cu, dtype=torch.int32, device=device)
         return self._cu_seqlens
+
+    def prompt_order(self, device) -> torch.Tensor:
+        """int32 [num_prompts] on the device: the prompts longest first (the order
+        their attention workgroups are started in), built once per step."""
+        if self._prompt_order is None or self._prompt_order.device != torch.device(device):
+            order = sorted(range(len(self.prompt_lens)), key=lambda i: -self.prompt_lens[i])
+            self._prompt_order = torch.tensor(order, dtype=torch.int32, device=device)
+        return self._prompt_order
 
 
 def build_cos_sin_cache(rotary_dim: int, max_position: int, base: float, device) -> torch.Tensor:
@@ -124,7 +133,8 @@ class PagedAttention(torch.nn.Module):
                                   num_tokens=n_valid)
         if n_prompt > 0:
             ops.prefill_causal(out[:n_prompt], query[:n_prompt], key[:n_prompt], value[:n_prompt],
-                               md.cu_seqlens(query.device), md.max_prompt_len, self.scale, self.num_kv_heads)
+                               md.cu_seqlens(query.device), md.max_prompt_len, self.scale, self.num_kv_heads,
+                               prompt_order=md.prompt_order(query.device))
         if md.num_generation_tokens > 0:
             if key_cache is None or value_cache is None:
                 raise ValueError("decode needs the KV pool")

@@ -68,6 +68,7 @@ struct PrefillParams {
   const uint16_t *q, *k, *v;
   int64_t out_stride, q_stride, kv_stride;
   const int32_t *cu_seqlens;
+  const int32_t *prompt_order;   // optional: prompts in the order their workgroups should start
   int32_t ratio;          // query heads per kv head
   int32_t q_tiles;        // 128-row query tiles per prompt (of the longest prompt)
   int32_t num_kv_heads;
@@ -109,7 +110,8 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
   const int group = (slot / per_group) * 8 + xcd;
   if (group >= P.num_groups) return;
   const int in_group = slot % per_group;
-  const int prompt = group / P.num_kv_heads;
+  const int prompt_rank = group / P.num_kv_heads;
+  const int prompt = P.prompt_order ? P.prompt_order[prompt_rank] : prompt_rank;
   const int hk = group % P.num_kv_heads;
   const int hq = hk * P.ratio + in_group / P.q_tiles;
   const int seq_begin = P.cu_seqlens[prompt];
@@ -443,9 +445,9 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
 
 extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const void *q, int64_t q_row_stride,
                                       const void *k, const void *v, int64_t kv_row_stride,
-                                      const int32_t *cu_seqlens, int32_t num_prompts, int32_t max_prompt_len,
-                                      int32_t num_q_heads, int32_t num_kv_heads, int32_t head_size,
-                                      float scale, int32_t dtype, void *stream) {
+                                      const int32_t *cu_seqlens, const int32_t *prompt_order, int32_t num_prompts,
+                                      int32_t max_prompt_len, int32_t num_q_heads, int32_t num_kv_heads,
+                                      int32_t head_size, float scale, int32_t dtype, void *stream) {
   using namespace mux;
   if (!out || !q || !k || !v || !cu_seqlens) return MUXA_EINVAL;
   if (num_prompts < 0 || max_prompt_len < 0 || num_q_heads <= 0 || num_kv_heads <= 0) return MUXA_EINVAL;
@@ -473,6 +475,7 @@ extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const v
   P.q_stride = q_row_stride;
   P.kv_stride = kv_row_stride;
   P.cu_seqlens = cu_seqlens;
+  P.prompt_order = prompt_order;
   P.ratio = num_q_heads / num_kv_heads;
   P.q_tiles = (max_prompt_len + kBM - 1) / kBM;
   P.num_kv_heads = num_kv_heads;

@@ -171,9 +171,18 @@ def paged_decode(out, q, k_pool, v_pool, block_tables, context_lens, max_context
 
 
 def prefill_causal(out, q, k, v, cu_seqlens: torch.Tensor, max_prompt_len: int, scale: float,
-                   num_kv_heads: int, stream=None) -> None:
-    """Causal attention over packed prompts; cu_seqlens int32 [P+1] on the device."""
+                   num_kv_heads: int, stream=None, prompt_order: Optional[torch.Tensor] = None) -> None:
+    """Causal attention over packed prompts; cu_seqlens int32 [P+1] on the device.
+    prompt_order: optional int32 [P] on the device, the prompts longest first
+    (scheduling only; results are the same)."""
     _need_cuda(out, q, k, v, cu_seqlens)
+    order_ptr = None
+    if prompt_order is not None:
+        _need_cuda(prompt_order)
+        if prompt_order.dtype != torch.int32 or prompt_order.dim() != 1 or not prompt_order.is_contiguous() \
+                or prompt_order.shape[0] != cu_seqlens.shape[0] - 1:
+            raise ValueError("prompt_order: expected contiguous int32 [P]")
+        order_ptr = prompt_order.data_ptr()
     if cu_seqlens.dtype != torch.int32 or cu_seqlens.dim() != 1 or not cu_seqlens.is_contiguous():
         raise ValueError("cu_seqlens: expected contiguous int32 [P+1]")
     if q.shape[1] % HEAD_SIZE or k.shape[1] != num_kv_heads * HEAD_SIZE or k.shape != v.shape:
@@ -185,7 +194,7 @@ def prefill_causal(out, q, k, v, cu_seqlens: torch.Tensor, max_prompt_len: int, 
         raise ValueError("k and v row strides differ")
     rc = _lib.attn().mux_prefill_causal(
         out.data_ptr(), _rows(out, "out"), q.data_ptr(), _rows(q, "q"), k.data_ptr(), v.data_ptr(), kv_stride,
-        cu_seqlens.data_ptr(), cu_seqlens.shape[0] - 1, int(max_prompt_len), q.shape[1] // HEAD_SIZE,
+        cu_seqlens.data_ptr(), order_ptr, cu_seqlens.shape[0] - 1, int(max_prompt_len), q.shape[1] // HEAD_SIZE,
         int(num_kv_heads), HEAD_SIZE, float(scale), _dtype_code(q), _stream_ptr(stream))
     _lib.check_attn(rc, "mux_prefill_causal")
 

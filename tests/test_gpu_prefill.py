@@ -101,6 +101,33 @@ def test_prefill_long_prompt_and_unstrided_inputs():
     assert (got - want).abs().max().item() <= TOL
 
 
+def test_prefill_prompt_order_changes_scheduling_only():
+    """Longest-first, reversed and random start orders give bit-identical
+    outputs (each workgroup computes the same tile whichever order it starts in)."""
+    _announce("prefill prompt order")
+    rng = np.random.Generator(np.random.PCG64(12))
+    lens = [int(x) for x in rng.integers(1, 400, size=21)] + [0, 700]
+    T = sum(lens)
+    g = torch.Generator().manual_seed(12)
+    q = torch.randn((T, 6 * D), generator=g).half().to(DEV)
+    k = torch.randn((T, 3 * D), generator=g).half().to(DEV)
+    v = torch.randn((T, 3 * D), generator=g).half().to(DEV)
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32, device=DEV)
+    base = torch.zeros_like(q)
+    ops.prefill_causal(base, q, k, v, cu, max(lens), D ** -0.5, 3)
+    orders = [np.argsort(-np.asarray(lens), kind="stable"), np.arange(len(lens))[::-1].copy(),
+              rng.permutation(len(lens))]
+    for order in orders:
+        out = torch.zeros_like(q)
+        ops.prefill_causal(out, q, k, v, cu, max(lens), D ** -0.5, 3,
+                           prompt_order=torch.from_numpy(order.astype(np.int32)).to(DEV))
+        torch.cuda.synchronize()
+        assert torch.equal(out, base)
+    with pytest.raises(ValueError):
+        ops.prefill_causal(base, q, k, v, cu, max(lens), D ** -0.5, 3,
+                           prompt_order=torch.zeros((3,), dtype=torch.int32, device=DEV))
+
+
 def test_prefill_first_token_and_block_diagonal_properties():
     """Row 0 of every prompt equals its own v; changing one prompt's k leaves
     every other prompt's output bit-identical."""
