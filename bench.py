@@ -56,7 +56,7 @@ def parse():
                     help="prefill3: start the prompts' workgroups as packed instead of longest first")
     ap.add_argument("--unfused", action="store_true", help="one launch per model instead of one fused launch")
     ap.add_argument("--workload", default="mixed3_decode",
-                    choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long", "model_ops"],
+                    choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long", "model_ops", "host_step"],
                     help="mixed3_decode is the headline metric; the others are the remaining synthetic "
                          "shapes, each printing its own JSON line")
     return ap.parse_args()
@@ -379,6 +379,92 @@ def bench_model_ops(args):
                  cfg, roof)
 
 
+def _host_step(sched, storage, L, H, ids, last_tokens, permuted):
+    """One step of the host path with the reference's call sequence
+    (llm_runtime.py:277-339): try_batch -> allocate_batch -> get_batch_info ->
+    caller-allocated CPU tensors -> get_batch.  Works with the product's classes
+    and with the compiled reference's."""
+    import torch
+    info = np.asarray(sched.try_batch(list(ids), list(last_tokens)), dtype=np.int32)
+    req = np.ascontiguousarray(info[:-1])
+    if int(info[-1]) > 0:
+        block_info = np.asarray(storage.allocate_batch(req, L, H), dtype=np.int32)
+    else:
+        block_info = np.array([len(ids)], dtype=np.int32)
+    bi = list(sched.get_batch_info(req, block_info))
+    T, C, max_ctx, max_blk = bi[:4]
+    slots = torch.empty((T, L, H), dtype=torch.int64)
+    toks = torch.empty(((T + 7) // 8 * 8,), dtype=torch.int32)
+    pos = torch.empty_like(toks)
+    ctx = torch.empty((C,), dtype=torch.int32)
+    if max_ctx > 0 and permuted:
+        tables = torch.empty((L, C, H, max_blk), dtype=torch.int32)
+        sched.get_batch_permuted(req, block_info, toks, pos, ctx, tables, slots)
+    else:
+        tables = torch.empty((T, max_blk, L, H) if max_ctx > 0 else (0, max_blk, 0, 0), dtype=torch.int32)
+        sched.get_batch(req, block_info, toks, pos, ctx, tables, slots)
+        if max_ctx > 0:
+            tables = tables.permute(2, 0, 3, 1).contiguous()        # llm_runtime.py:327 (on the device there)
+    return tables, slots
+
+
+def _time_host(make_storage, make_sched, L, H, lens, decode_steps, permuted):
+    """(prefill step seconds, mean decode step seconds) for one batch."""
+    bs = 16
+    need = sum((n + decode_steps + bs) // bs + 1 for n in lens) * L * H
+    storage, sched = make_storage(need + 1024), make_sched(L, H, 2048, bs)
+    rng = np.random.Generator(np.random.PCG64(1))
+    ids = list(range(len(lens)))
+    for i, n in enumerate(lens):
+        sched.add_request(rng.integers(0, 32000, size=int(n)).astype(np.int32), i, decode_steps + 8)
+    t0 = time.perf_counter()
+    _host_step(sched, storage, L, H, ids, [], permuted)
+    t1 = time.perf_counter()
+    for s in range(decode_steps):
+        _host_step(sched, storage, L, H, ids, [7 + s] * len(ids), permuted)
+    t2 = time.perf_counter()
+    return t1 - t0, (t2 - t1) / decode_steps
+
+
+def bench_host_step(args):
+    """The host side of a step at real layer counts, single-threaded as in the
+    reference: the product's allocator + batch builder, and beside it the
+    reference's own C++ compiled under oracle/_ref when that is present."""
+    from muxserve_amd.batch_scheduler import BatchScheduler
+    from muxserve_amd.memory_manager import KVStorage
+    rng = np.random.Generator(np.random.PCG64(args.seed))
+    shapes = {"7b (L32,H32), 32 sequences": (32, 32, 32), "13b (L40,H40), 16 sequences": (40, 40, 16),
+              "30b (L60,H52), 8 sequences": (60, 52, 8)}
+    ref = (None, None)
+    if not args.no_cpu_baseline:
+        from oracle import build_ref                                  # the checker: CPU baseline only
+        if os.path.isdir(os.path.join(ROOT, "oracle", "_ref")):
+            ref = build_ref.load()
+    steps = 64
+    rows, total_dec, total_ref = {}, 0.0, 0.0
+    for name, (L, H, B) in shapes.items():
+        lens = np.clip(np.rint(rng.lognormal(np.log(300), 0.8, size=B)), 16, 1900).astype(int)
+        pre_p, dec_p = _time_host(KVStorage, BatchScheduler, L, H, lens, steps, True)
+        pre_l, dec_l = _time_host(KVStorage, BatchScheduler, L, H, lens, steps, False)
+        row = {"prefill_step_ms": pre_p * 1e3, "decode_step_us": dec_p * 1e6,
+               "decode_step_us_reference_layout_then_permute": dec_l * 1e6}
+        total_dec += dec_p
+        if ref[0] is not None:
+            pre_r, dec_r = _time_host(ref[0].KVStorage, ref[1].BatchScheduler, L, H, lens, steps, False)
+            row["reference_prefill_step_ms"] = pre_r * 1e3
+            row["reference_decode_step_us"] = dec_r * 1e6
+            total_ref += dec_r
+        rows[name] = row
+    line = _line("host path: decode step of the three models, microseconds", total_dec * 1e6, "us", args,
+                 total_dec * 1e3, {"workload": "host_step", "decode_steps_timed": steps, "threads": 1, "models": rows},
+                 None, dtype="int32", higher=False)
+    if ref[0] is not None:
+        line["cpu_baseline"] = {"value": total_ref * 1e6, "unit": "us", "cores": 1, "kind": "reference",
+                                "sample": f"the same {steps} decode steps through the reference's compiled "
+                                          "memory_manager / batch_scheduler, table permuted on the host"}
+    return line
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -386,7 +472,7 @@ def main():
               file=sys.stderr)
         sys.exit(2)
     other = {"prefill3": bench_prefill3, "cache_write": bench_cache_write, "colocated": bench_colocated,
-             "gqa_long": bench_gqa_long, "model_ops": bench_model_ops}
+             "gqa_long": bench_gqa_long, "model_ops": bench_model_ops, "host_step": bench_host_step}
     if args.workload in other:
         print(json.dumps(other[args.workload](args)))
         return

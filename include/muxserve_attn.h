@@ -234,6 +234,29 @@ int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_states, int64
                           int32_t hidden_size, int32_t dtype, void *workspace, size_t workspace_bytes,
                           void *stream);
 
+/* ---- Step inputs built on the device ---------------------------------------
+ * No reference counterpart (the reference builds slot_mapping and the block
+ * table on the host, csrc/batch_scheduler.cpp:131-169, and uploads them,
+ * muxserve/flexserver/llm_runtime.py:301-327).  Companion of
+ * mux_sched_get_batch_compact (muxserve_host.h): mirror is a DEVICE int32
+ * [max_rows, max_blocks_per_seq, L, H] array the caller allocates once and
+ * only this call writes; desc (DEVICE int32 [num_seqs, 8]) and block_info
+ * (DEVICE copy of the allocator's reply, n_block_info ints) are the step's
+ * upload.  In stream order: the reply's ids are appended to the mirror rows,
+ * slot_mapping int64 [num_tokens, L, H] is written, and, when
+ * max_blocks_out > 0 (decode step), block_tables int32
+ * [L, num_seqs, H, max_blocks_out] - both bit-identical to what
+ * mux_sched_get_batch + permute(2,0,3,1) give on the entries the reference
+ * defines (others 0).  max_new_blocks: host-side upper bound of desc[.][3]
+ * (sizes the copy grid).  Descriptors that do not fit the mirror or the reply
+ * are skipped. */
+int32_t mux_build_step_inputs(int32_t *mirror, int32_t max_rows, int32_t max_blocks_per_seq,
+                              int32_t num_layers, int32_t num_heads, int32_t block_size,
+                              const int32_t *desc, int32_t num_seqs, const int32_t *block_info,
+                              int64_t n_block_info, int32_t max_new_blocks, int32_t num_tokens,
+                              int64_t *slot_mapping, int32_t *block_tables, int32_t max_blocks_out,
+                              void *stream);
+
 /* ---- CU-masked streams ---------------------------------------------------
  * Replacement for the reference's per-process MPS share
  * (CUDA_MPS_ACTIVE_THREAD_PERCENTAGE, muxserve/muxsched/launcher.py:54-61):

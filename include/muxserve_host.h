@@ -122,6 +122,36 @@ int64_t mux_sched_get_batch_permuted(MuxBatchScheduler *s, const int32_t *req, i
                                      int32_t max_blocks,
                                      int64_t *slot_mapping, int64_t slot_mapping_cap);
 
+/* No reference counterpart: the step without the O(tokens x L x H) host work.
+ * The reference rebuilds the whole block table and a slot per (token, layer,
+ * head) on the host every step and uploads both (csrc/batch_scheduler.cpp:
+ * 131-169, muxserve/flexserver/llm_runtime.py:301-327: 16 MB of table per
+ * decode step of a 7B model, 130 MB of slots per prefill step of a 30B model).
+ * Here the device keeps a mirror of every request's id run
+ * [row][token block][L][H]; a step uploads only the allocator's reply and
+ * MUX_STEP_DESC_INTS ints per sequence, and mux_build_step_inputs
+ * (muxserve_attn.h) derives slot_mapping and the step's block table on the
+ * device, bit-identical to what mux_sched_get_batch writes.
+ *
+ * mux_sched_enable_device_rows: once, before the first compact step; max_rows =
+ * rows of the device mirror (>= requests alive at a time).
+ * mux_sched_get_batch_compact: same step protocol and side effects as
+ * mux_sched_get_batch (preempted requests forgotten, prompt_info / batch_reqs
+ * refreshed, tokens / positions / context_lens filled); instead of tables and
+ * slots it writes one descriptor per batch entry i < block_info[0]:
+ *   desc[i] = { row, numPhysicalBlocks, first token block brought by this
+ *               reply, token blocks brought, offset of their ids in block_info,
+ *               contextLen (decode) or promptLen, first token of the entry in
+ *               the batch, 1 if decoding }
+ * MUX_ENOSPC when no row is free.  Returns numTokens. */
+#define MUX_STEP_DESC_INTS 8
+int32_t mux_sched_enable_device_rows(MuxBatchScheduler *s, int32_t max_rows);
+int64_t mux_sched_get_batch_compact(MuxBatchScheduler *s, const int32_t *req, int32_t n_req,
+                                    const int32_t *block_info, int64_t n_block_info,
+                                    int32_t *tokens, int32_t *positions, int64_t n_tok_padded,
+                                    int32_t *context_lens, int64_t context_lens_cap,
+                                    int32_t *desc, int64_t desc_cap);
+
 /* BatchScheduler::releaseRequests, csrc/batch_scheduler.cpp:195-199. */
 int32_t mux_sched_release_requests(MuxBatchScheduler *s, const int32_t *request_ids, int32_t n);
 

@@ -58,6 +58,9 @@ def host():
                                         c_vp, c_i64, c_vp, c_i64, c_vp, c_i64]),
         "mux_sched_get_batch_permuted": (c_i64, [c_vp, c_vp, c_i32, c_vp, c_i64, c_vp, c_vp, c_i64,
                                                  c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_i64]),
+        "mux_sched_enable_device_rows": (c_i32, [c_vp, c_i32]),
+        "mux_sched_get_batch_compact": (c_i64, [c_vp, c_vp, c_i32, c_vp, c_i64, c_vp, c_vp, c_i64,
+                                                c_vp, c_i64, c_vp, c_i64]),
         "mux_sched_release_requests": (c_i32, [c_vp, c_vp, c_i32]),
         "mux_sched_get_preempt_requests": (c_i32, [c_vp, c_vp, c_i32]),
         "mux_sched_get_prompt_info": (c_i32, [c_vp, c_vp, c_i32]),
@@ -135,6 +138,8 @@ ATTN_SIGNATURES = {
     "mux_greedy_sample_workspace_init": (c_i32, [c_vp, c_sz, c_vp]),
     "mux_greedy_sample": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_i32, c_vp, c_i64, c_i32, c_i32, c_i32, c_i32,
                                   c_vp, c_sz, c_vp]),
+    "mux_build_step_inputs": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_i32, c_vp, c_i64, c_i32,
+                                      c_i32, c_vp, c_vp, c_i32, c_vp]),
     "mux_stream_create_cu_range": (c_i32, [c_vp, c_i32, c_i32, c_vp]),
     "mux_stream_destroy": (c_i32, [c_vp]),
     "mux_device_cu_info": (c_i32, [c_vp]),

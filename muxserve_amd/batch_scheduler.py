@@ -112,6 +112,31 @@ class BatchScheduler:
                                                                max_blocks, slot, n_slot),
                         "BatchScheduler.get_batch_permuted")
 
+    STEP_DESC_INTS = 8
+
+    def enable_device_rows(self, max_rows: int) -> None:
+        """Not in the reference: switch on the bookkeeping for a device-resident
+        mirror of the requests' block-id runs (see get_batch_compact)."""
+        _lib.check_host(self._lib.mux_sched_enable_device_rows(self._h, int(max_rows)),
+                        "BatchScheduler.enable_device_rows")
+
+    def get_batch_compact(self, batch_info, block_info, token_tensor, token_position_tensor,
+                          context_len_tensor, desc_tensor) -> None:
+        """Not in the reference: get_batch without the block table and the slot
+        mapping; instead one row of STEP_DESC_INTS int32 per batch entry goes to
+        desc_tensor, from which the device builds both."""
+        req, blk = _i32(batch_info), _i32(block_info)
+        tok, n_tok = _buf(token_tensor, np.int32, "token_tensor")
+        pos, n_pos = _buf(token_position_tensor, np.int32, "token_position_tensor")
+        ctx, n_ctx = _buf(context_len_tensor, np.int32, "context_len_tensor")
+        desc, n_desc = _buf(desc_tensor, np.int32, "desc_tensor")
+        if n_pos != n_tok:
+            raise ValueError("token and position tensors must have the same length")
+        _lib.check_host(self._lib.mux_sched_get_batch_compact(self._h, req.ctypes.data, req.size,
+                                                              blk.ctypes.data, blk.size,
+                                                              tok, pos, n_tok, ctx, n_ctx, desc, n_desc),
+                        "BatchScheduler.get_batch_compact")
+
     def release_requests(self, request_ids) -> None:
         ids = _i32(list(request_ids))
         _lib.check_host(self._lib.mux_sched_release_requests(self._h, ids.ctypes.data, ids.size),

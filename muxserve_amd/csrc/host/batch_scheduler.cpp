@@ -30,6 +30,7 @@ struct Sequence {
   std::vector<int32_t> prompt;
   std::vector<int32_t> outputs;
   std::vector<int32_t> ids;      // [physical_blocks][L][H]
+  int32_t row = -1;              // row of the device-resident table mirror, once assigned
 
   bool decoding() const { return !outputs.empty(); }
 };
@@ -40,10 +41,20 @@ struct MuxBatchScheduler {
   int32_t L = 0, H = 0, max_seq_len = 0, block_size = 0, max_blocks_per_seq = 0;
   std::unordered_map<int32_t, std::unique_ptr<Sequence>> seqs;
   std::vector<int32_t> preempted, prompt_info, batch_reqs;
+  std::vector<int32_t> free_rows;            // device-table rows not in use (empty: feature off)
+  int32_t max_rows = 0;
 
   Sequence *find(int32_t id) const {
     auto it = seqs.find(id);
     return it == seqs.end() ? nullptr : it->second.get();
+  }
+  // Forget a request; its device-table row goes back to the free list.
+  int32_t drop(int32_t id) {
+    auto it = seqs.find(id);
+    if (it == seqs.end()) return 0;
+    if (it->second->row >= 0) free_rows.push_back(it->second->row);
+    seqs.erase(it);
+    return 1;
   }
 };
 
@@ -115,7 +126,7 @@ int64_t fill_batch(MuxBatchScheduler *s, const int32_t *req, int32_t n_req,
     const int32_t id = req[3 * i];
     if (i >= cut) {     // preempted by the allocator: forget the request
       s->preempted.push_back(id);
-      s->seqs.erase(id);
+      s->drop(id);
       continue;
     }
     Sequence *q = s->find(id);
@@ -212,7 +223,8 @@ int32_t mux_sched_add_request(MuxBatchScheduler *s, const int32_t *prompt, int32
   // (C++ truncating division, so an empty prompt gives block -1, offset -1).
   q->logical_block = (prompt_len + s->block_size - 1) / s->block_size - 1;
   q->logical_offset = (prompt_len - 1) % s->block_size;
-  s->seqs[req_id] = std::move(q);   // re-adding an id replaces the old request
+  s->drop(req_id);                  // re-adding an id replaces the old request
+  s->seqs[req_id] = std::move(q);
   return MUX_OK;
 }
 
@@ -322,10 +334,112 @@ int64_t mux_sched_get_batch_permuted(MuxBatchScheduler *s, const int32_t *req, i
                     /*permuted=*/true, max_blocks, slot_mapping, slot_mapping_cap);
 }
 
+int32_t mux_sched_enable_device_rows(MuxBatchScheduler *s, int32_t max_rows) {
+  if (!s || max_rows <= 0) return MUX_EINVAL;
+  if (s->max_rows != 0) return MUX_ESTATE;
+  s->max_rows = max_rows;
+  s->free_rows.resize(static_cast<size_t>(max_rows));
+  for (int32_t r = 0; r < max_rows; ++r) s->free_rows[static_cast<size_t>(r)] = max_rows - 1 - r;   // row 0 first
+  return MUX_OK;
+}
+
+int64_t mux_sched_get_batch_compact(MuxBatchScheduler *s, const int32_t *req, int32_t n_req,
+                                    const int32_t *block_info, int64_t n_block_info,
+                                    int32_t *tokens, int32_t *positions, int64_t n_tok_padded,
+                                    int32_t *context_lens, int64_t context_lens_cap,
+                                    int32_t *desc, int64_t desc_cap) {
+  if (!s || !req || !block_info || n_req < 0 || n_block_info < 1 || n_tok_padded < 0) return MUX_EINVAL;
+  if (s->max_rows == 0) return MUX_ESTATE;
+  const int32_t rows = n_req / 3;
+  const int32_t cut = block_info[0];
+  const int64_t per = static_cast<int64_t>(s->L) * s->H;
+  const int32_t bs = s->block_size;
+
+  // Pass 1 (read-only): sizes and row demand, checked before any write or drop.
+  int64_t n_tokens = 0, n_ctx = 0, n_live = 0, new_rows = 0, freed_rows = 0;
+  for (int32_t i = 0; i < rows; ++i) {
+    const Sequence *q = s->find(req[3 * i]);
+    if (i >= cut) {
+      if (q && q->row >= 0) ++freed_rows;
+      continue;
+    }
+    if (!q) return MUX_ENOENT;
+    if (q->physical_blocks > s->max_blocks_per_seq) return MUX_ENOSPC;
+    if (q->decoding()) {
+      if (q->physical_blocks < 1) return MUX_ESTATE;
+      n_tokens += 1;
+      n_ctx += 1;
+    } else {
+      const int64_t p = static_cast<int64_t>(q->prompt.size());
+      if ((p + bs - 1) / bs > q->physical_blocks) return MUX_ESTATE;
+      n_tokens += p;
+    }
+    if (q->row < 0) ++new_rows;
+    ++n_live;
+  }
+  if (n_tokens > n_tok_padded || n_ctx > context_lens_cap || n_live * MUX_STEP_DESC_INTS > desc_cap) return MUX_ENOSPC;
+  if (new_rows > static_cast<int64_t>(s->free_rows.size()) + freed_rows) return MUX_ENOSPC;
+  if ((n_tokens > 0 && (!tokens || !positions)) || (n_ctx > 0 && !context_lens) || (n_live > 0 && !desc))
+    return MUX_EINVAL;
+
+  // Pass 2: requests the allocator preempted go first (their rows become free).
+  s->preempted.clear();
+  s->prompt_info.clear();
+  s->batch_reqs.clear();
+  for (int32_t i = std::max(cut, 0); i < rows; ++i) {
+    s->preempted.push_back(req[3 * i]);
+    s->drop(req[3 * i]);
+  }
+  int64_t t = 0, c = 0, cursor = 1;
+  int32_t max_ctx = 0;
+  for (int32_t i = 0; i < rows && i < cut; ++i) {
+    Sequence *q = s->find(req[3 * i]);
+    if (q->row < 0) {
+      q->row = s->free_rows.back();
+      s->free_rows.pop_back();
+    }
+    const int32_t granted = std::max(req[3 * i + 1], 0);
+    int32_t *d = desc + static_cast<int64_t>(i) * MUX_STEP_DESC_INTS;
+    d[0] = q->row;
+    d[1] = q->physical_blocks;
+    d[2] = q->physical_blocks - granted;          // first token block the reply brought
+    d[3] = granted;
+    d[4] = static_cast<int32_t>(cursor);           // where its ids start in block_info
+    d[6] = static_cast<int32_t>(t);
+    cursor += static_cast<int64_t>(granted) * per;
+    if (q->decoding()) {
+      tokens[t] = q->outputs.back();
+      positions[t] = q->context_len - 1;
+      context_lens[c] = q->context_len;
+      max_ctx = std::max(max_ctx, q->context_len);
+      d[5] = q->context_len;
+      d[7] = 1;
+      t += 1;
+      c += 1;
+    } else {
+      const int64_t p = static_cast<int64_t>(q->prompt.size());
+      std::memcpy(tokens + t, q->prompt.data(), sizeof(int32_t) * static_cast<size_t>(p));
+      for (int64_t k = 0; k < p; ++k) positions[t + k] = static_cast<int32_t>(k);
+      s->prompt_info.push_back(static_cast<int32_t>(p));
+      d[5] = static_cast<int32_t>(p);
+      d[7] = 0;
+      t += p;
+    }
+    s->batch_reqs.push_back(q->id);
+    s->batch_reqs.push_back(q->max_tokens);
+  }
+  s->prompt_info.push_back(max_ctx);
+  for (int64_t k = t; k < n_tok_padded; ++k) {
+    tokens[k] = 0;
+    positions[k] = 0;
+  }
+  return n_tokens;
+}
+
 int32_t mux_sched_release_requests(MuxBatchScheduler *s, const int32_t *request_ids, int32_t n) {
   if (!s || n < 0 || (n > 0 && !request_ids)) return MUX_EINVAL;
   int32_t erased = 0;
-  for (int32_t i = 0; i < n; ++i) erased += static_cast<int32_t>(s->seqs.erase(request_ids[i]));
+  for (int32_t i = 0; i < n; ++i) erased += s->drop(request_ids[i]);
   return erased;
 }
 

@@ -13,6 +13,7 @@ from oracle import attn_oracle as orc
 from muxserve_amd import ops
 from muxserve_amd.attention import PagedAttentionWithRoPE
 from muxserve_amd.batch_scheduler import BatchScheduler
+from muxserve_amd.device_tables import DeviceBlockTables
 from muxserve_amd.memory_manager import KVStorage
 from muxserve_amd.pool import HEAD_SIZE, allocate_gpu_cache
 from muxserve_amd.prepare import prepare_inputs
@@ -24,7 +25,7 @@ TOL = 2e-3
 
 
 class _Model:
-    def __init__(self, name, L, Hq, Hkv, storage, bs, seed, fused_rope_max_tokens=512):
+    def __init__(self, name, L, Hq, Hkv, storage, bs, seed, fused_rope_max_tokens=512, device_rows=0):
         self.name, self.L, self.Hq, self.Hkv = name, L, Hq, Hkv
         self.sched = BatchScheduler(L, Hkv, 512, bs)
         self.storage = storage
@@ -33,6 +34,7 @@ class _Model:
         for layer in self.layers:
             layer.fused_rope_max_tokens = fused_rope_max_tokens
         self.g = torch.Generator().manual_seed(seed)
+        self.device_tables = DeviceBlockTables(self.sched, device_rows, DEV) if device_rows else None
 
     def alloc(self, req):
         return self.storage.allocate_batch(req, self.L, self.Hkv)
@@ -40,7 +42,8 @@ class _Model:
 
 def _step(m, ids, last_tokens, k_pool, v_pool, hk, hv, permuted):
     tokens, positions, md, batch_reqs, preempted = prepare_inputs(m.sched, m.alloc, ids, last_tokens, DEV,
-                                                                  permuted_tables=permuted)
+                                                                  permuted_tables=permuted,
+                                                                  device_tables=m.device_tables)
     assert not preempted
     T_pad = tokens.shape[0]
     n = md.num_valid_tokens
@@ -72,19 +75,22 @@ def _step(m, ids, last_tokens, k_pool, v_pool, hk, hv, permuted):
     return worst
 
 
-@pytest.mark.parametrize("permuted,fused_max", [(True, 512), (False, 512), (True, 0), (True, 60)])
-def test_two_models_share_one_pool_prefill_then_decode(permuted, fused_max):
+@pytest.mark.parametrize("permuted,fused_max,device_rows", [(True, 512, 0), (False, 512, 0), (True, 0, 0),
+                                                            (True, 60, 0), (True, 512, 8)])
+def test_two_models_share_one_pool_prefill_then_decode(permuted, fused_max, device_rows):
     """fused_max: steps of up to that many tokens rotate and write the cache in
-    one launch (0: always the two kernels; 60: decode steps fused, prefill not)."""
-    print(f"[case] serving path permuted_tables={permuted} fused_rope_max_tokens={fused_max}", flush=True)
+    one launch (0: always the two kernels; 60: decode steps fused, prefill not).
+    device_rows > 0: slot mapping and block tables are built on the device."""
+    print(f"[case] serving path permuted_tables={permuted} fused_rope_max_tokens={fused_max} "
+          f"device_rows={device_rows}", flush=True)
     bs, N = 16, 6000
     storage = KVStorage(N)
     k_pool, v_pool = allocate_gpu_cache(N, bs, DEV)
     k_pool.zero_()
     v_pool.zero_()
     hk, hv = k_pool.cpu(), v_pool.cpu()
-    a = _Model("small-mha", 2, 4, 4, storage, bs, seed=1, fused_rope_max_tokens=fused_max)
-    b = _Model("gqa", 3, 8, 2, storage, bs, seed=2, fused_rope_max_tokens=fused_max)
+    a = _Model("small-mha", 2, 4, 4, storage, bs, seed=1, fused_rope_max_tokens=fused_max, device_rows=device_rows)
+    b = _Model("gqa", 3, 8, 2, storage, bs, seed=2, fused_rope_max_tokens=fused_max, device_rows=device_rows)
     rng = np.random.Generator(np.random.PCG64(3))
     for m, lens, base_id in ((a, [5, 40, 17], 0), (b, [130, 16, 1, 33], 100)):
         for i, p in enumerate(lens):

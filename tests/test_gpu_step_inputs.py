@@ -1,0 +1,93 @@
+"""prepare_inputs with the device-side builder (DeviceBlockTables) against
+prepare_inputs on the reference-shaped host path: the same scenario is driven
+through two scheduler/allocator pairs in lockstep and every tensor the model
+code receives must be bit-identical (block-table entries the reference leaves
+undefined excepted)."""
+import numpy as np
+import pytest
+import torch
+
+from muxserve_amd.batch_scheduler import BatchScheduler
+from muxserve_amd.device_tables import DeviceBlockTables
+from muxserve_amd.memory_manager import KVStorage
+from muxserve_amd.prepare import prepare_inputs
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _pair(L, H, bs, N, rows, max_seq_len=1024):
+    a = (KVStorage(N), BatchScheduler(L, H, max_seq_len, bs))
+    b = (KVStorage(N), BatchScheduler(L, H, max_seq_len, bs))
+    dt = DeviceBlockTables(b[1], rows, DEV)
+    return a, b, dt
+
+
+def _both(a, b, dt, L, H, ids, last, bs):
+    ra = prepare_inputs(a[1], lambda r: a[0].allocate_batch(r, L, H), ids, last, DEV, permuted_tables=False)
+    rb = prepare_inputs(b[1], lambda r: b[0].allocate_batch(r, L, H), ids, last, DEV, device_tables=dt)
+    torch.cuda.synchronize()
+    (ta, pa, ma, qa, ea), (tb, pb, mb, qb, eb) = ra, rb
+    assert torch.equal(ta, tb) and torch.equal(pa, pb) and qa == qb and ea == eb
+    assert ma.prompt_lens == mb.prompt_lens and ma.max_context_len == mb.max_context_len
+    assert ma.total_context_len == mb.total_context_len
+    assert torch.equal(ma.context_lens, mb.context_lens)
+    assert ma.slot_mapping.shape == mb.slot_mapping.shape and torch.equal(ma.slot_mapping, mb.slot_mapping)
+    if ma.max_context_len > 0:
+        assert ma.block_tables.shape == mb.block_tables.shape
+        xa, xb = ma.block_tables.cpu(), mb.block_tables.cpu()
+        for c, n in enumerate(ma.context_lens.cpu().tolist()):
+            valid = (n + bs - 1) // bs
+            assert torch.equal(xa[:, c, :, :valid], xb[:, c, :, :valid]), f"sequence {c}"
+    else:
+        assert mb.block_tables.numel() == 0
+    return ea
+
+
+@pytest.mark.parametrize("L,H,bs", [(2, 4, 16), (32, 32, 16), (3, 5, 8), (60, 52, 16), (1, 1, 32)])
+def test_device_built_step_inputs_equal_the_host_built_ones(L, H, bs):
+    print(f"[case] device step inputs L={L} H={H} bs={bs}", flush=True)
+    rng = np.random.Generator(np.random.PCG64(L + H))
+    lens = [int(x) for x in rng.integers(1, 200, size=7)] + [bs, 2 * bs + 1]
+    N = (sum((n + 40) // bs + 2 for n in lens)) * L * H + 256
+    a, b, dt = _pair(L, H, bs, N, rows=12)
+    for i, p in enumerate(lens):
+        prompt = rng.integers(0, 32000, size=p).astype(np.int32)
+        a[1].add_request(prompt, i, 64)
+        b[1].add_request(prompt, i, 64)
+    ids = list(range(len(lens)))
+    _both(a, b, dt, L, H, ids[:5], [], bs)                         # two prefill steps
+    _both(a, b, dt, L, H, ids[5:], [], bs)
+    for step in range(bs + 3):                                      # decode across block boundaries
+        order = ids[::-1] if step % 2 else ids
+        _both(a, b, dt, L, H, order, [step + 1] * len(ids), bs)
+    for st, sc in (a, b):                                           # release, then new requests reuse rows
+        st.free_batch([0, 4, 8])
+        sc.release_requests([0, 4, 8])
+    for rid, p in ((20, 33), (21, 1), (22, 3 * bs)):
+        prompt = rng.integers(0, 32000, size=p).astype(np.int32)
+        a[1].add_request(prompt, rid, 64)
+        b[1].add_request(prompt, rid, 64)
+    _both(a, b, dt, L, H, [20, 21, 22], [], bs)
+    live = [1, 2, 3, 5, 6, 7, 20, 21, 22]
+    for step in range(4):
+        _both(a, b, dt, L, H, live, [9] * len(live), bs)
+
+
+def test_device_built_step_inputs_with_preemption():
+    print("[case] device step inputs, preemption", flush=True)
+    L, H, bs = 2, 2, 16
+    N = 10 * L * H
+    a, b, dt = _pair(L, H, bs, N, rows=4, max_seq_len=256)
+    for i, p in enumerate([3 * bs, 3 * bs, 2 * bs + 5, 2 * bs]):
+        prompt = np.arange(p, dtype=np.int32)
+        a[1].add_request(prompt, i, 32)
+        b[1].add_request(prompt, i, 32)
+    cut = _both(a, b, dt, L, H, [0, 1, 2, 3], [], bs)
+    assert cut, "the pool was meant to be too small for the batch"
+    alive = [r for r in [0, 1, 2, 3] if r not in cut]
+    for step in range(2 * bs):
+        cut = _both(a, b, dt, L, H, alive, [3] * len(alive), bs)
+        alive = [r for r in alive if r not in cut]
+        if not alive:
+            break
