@@ -408,8 +408,32 @@ def _host_step(sched, storage, L, H, ids, last_tokens, permuted):
     return tables, slots
 
 
-def _time_host(make_storage, make_sched, L, H, lens, decode_steps, permuted):
-    """(prefill step seconds, mean decode step seconds) for one batch."""
+def _host_step_compact(sched, storage, L, H, ids, last_tokens, staging):
+    """The host part of a step when the device builds the tables: the same
+    calls up to get_batch_info, then 8 ints per sequence instead of tables and
+    slots, everything packed into one staging buffer."""
+    import torch
+    info = np.asarray(sched.try_batch(list(ids), list(last_tokens)), dtype=np.int32)
+    req = np.ascontiguousarray(info[:-1])
+    if int(info[-1]) > 0:
+        block_info = np.asarray(storage.allocate_batch(req, L, H), dtype=np.int32)
+    else:
+        block_info = np.array([len(ids)], dtype=np.int32)
+    bi = list(sched.get_batch_info(req, block_info))
+    T, C = bi[:2]
+    pad = (T + 7) // 8 * 8
+    n = max(int(block_info[0]), 0)
+    o_ctx, o_desc = 2 * pad, 2 * pad + (C + 3) // 4 * 4
+    o_info = o_desc + 8 * n
+    sched.get_batch_compact(req, block_info, staging[:pad], staging[pad:o_ctx], staging[o_ctx:o_ctx + C],
+                            staging[o_desc:o_info])
+    staging[o_info:o_info + block_info.size] = torch.from_numpy(block_info)
+    return o_info + block_info.size
+
+
+def _time_host(make_storage, make_sched, L, H, lens, decode_steps, permuted, compact=False):
+    """(prefill step seconds, mean decode step seconds[, ints uploaded per decode step]) for one batch."""
+    import torch
     bs = 16
     need = sum((n + decode_steps + bs) // bs + 1 for n in lens) * L * H
     storage, sched = make_storage(need + 1024), make_sched(L, H, 2048, bs)
@@ -417,11 +441,54 @@ def _time_host(make_storage, make_sched, L, H, lens, decode_steps, permuted):
     ids = list(range(len(lens)))
     for i, n in enumerate(lens):
         sched.add_request(rng.integers(0, 32000, size=int(n)).astype(np.int32), i, decode_steps + 8)
+    if compact:
+        sched.enable_device_rows(len(lens))
+        staging = torch.empty((need + 65536,), dtype=torch.int32)
+        t0 = time.perf_counter()
+        _host_step_compact(sched, storage, L, H, ids, [], staging)
+        t1 = time.perf_counter()
+        ints = 0
+        for s in range(decode_steps):
+            ints += _host_step_compact(sched, storage, L, H, ids, [7 + s] * len(ids), staging)
+        t2 = time.perf_counter()
+        return t1 - t0, (t2 - t1) / decode_steps, ints / decode_steps
     t0 = time.perf_counter()
     _host_step(sched, storage, L, H, ids, [], permuted)
     t1 = time.perf_counter()
     for s in range(decode_steps):
         _host_step(sched, storage, L, H, ids, [7 + s] * len(ids), permuted)
+    t2 = time.perf_counter()
+    return t1 - t0, (t2 - t1) / decode_steps
+
+
+def _time_prepare_inputs(L, H, lens, decode_steps, mode):
+    """Full prepare_inputs on the GPU box, wall clock per decode step including
+    uploads and kernels (synchronised at the end).  mode: "device" (tables and
+    slots built on the device), "lbhm" (host writes [L,B,H,maxBlk]) or
+    "reference" (host writes the reference layout, permuted on the device)."""
+    import torch
+    from muxserve_amd.batch_scheduler import BatchScheduler
+    from muxserve_amd.device_tables import DeviceBlockTables
+    from muxserve_amd.memory_manager import KVStorage
+    from muxserve_amd.prepare import prepare_inputs
+    bs = 16
+    need = sum((n + decode_steps + bs) // bs + 1 for n in lens) * L * H
+    storage, sched = KVStorage(need + 1024), BatchScheduler(L, H, 2048, bs)
+    kw = {"device_tables": DeviceBlockTables(sched, len(lens), "cuda:0")} if mode == "device" else \
+         {"permuted_tables": mode == "lbhm"}
+    rng = np.random.Generator(np.random.PCG64(1))
+    ids = list(range(len(lens)))
+    for i, n in enumerate(lens):
+        sched.add_request(rng.integers(0, 32000, size=int(n)).astype(np.int32), i, decode_steps + 8)
+    alloc = lambda r: storage.allocate_batch(r, L, H)   # noqa: E731
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    prepare_inputs(sched, alloc, ids, [], "cuda:0", **kw)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for s in range(decode_steps):
+        prepare_inputs(sched, alloc, ids, [7 + s] * len(ids), "cuda:0", **kw)
+    torch.cuda.synchronize()
     t2 = time.perf_counter()
     return t1 - t0, (t2 - t1) / decode_steps
 
@@ -441,21 +508,33 @@ def bench_host_step(args):
         if os.path.isdir(os.path.join(ROOT, "oracle", "_ref")):
             ref = build_ref.load()
     steps = 64
+    import torch
+    have_gpu = torch.cuda.is_available()
     rows, total_dec, total_ref = {}, 0.0, 0.0
     for name, (L, H, B) in shapes.items():
         lens = np.clip(np.rint(rng.lognormal(np.log(300), 0.8, size=B)), 16, 1900).astype(int)
         pre_p, dec_p = _time_host(KVStorage, BatchScheduler, L, H, lens, steps, True)
         pre_l, dec_l = _time_host(KVStorage, BatchScheduler, L, H, lens, steps, False)
-        row = {"prefill_step_ms": pre_p * 1e3, "decode_step_us": dec_p * 1e6,
-               "decode_step_us_reference_layout_then_permute": dec_l * 1e6}
-        total_dec += dec_p
+        pre_c, dec_c, ints = _time_host(KVStorage, BatchScheduler, L, H, lens, steps, True, compact=True)
+        row = {"compact_prefill_step_ms": pre_c * 1e3, "compact_decode_step_us": dec_c * 1e6,
+               "compact_upload_bytes_per_decode_step": 4 * ints,
+               "host_built_prefill_step_ms": pre_p * 1e3, "host_built_decode_step_us_lbhm": dec_p * 1e6,
+               "host_built_decode_step_us_reference_layout_then_permute": dec_l * 1e6,
+               "host_built_upload_bytes_per_decode_step":
+                   int(B * L * H * (8 + 4 * ((int(lens.max()) + steps) // 16 + 1)))}
+        if have_gpu:
+            for mode in ("device", "lbhm", "reference"):
+                pre_d, dec_d = _time_prepare_inputs(L, H, lens, steps, mode)
+                row[f"prepare_inputs_{mode}_prefill_ms"] = pre_d * 1e3
+                row[f"prepare_inputs_{mode}_decode_us"] = dec_d * 1e6
+        total_dec += dec_c
         if ref[0] is not None:
             pre_r, dec_r = _time_host(ref[0].KVStorage, ref[1].BatchScheduler, L, H, lens, steps, False)
             row["reference_prefill_step_ms"] = pre_r * 1e3
             row["reference_decode_step_us"] = dec_r * 1e6
             total_ref += dec_r
         rows[name] = row
-    line = _line("host path: decode step of the three models, microseconds", total_dec * 1e6, "us", args,
+    line = _line("host path (compact step): decode step of the three models, microseconds", total_dec * 1e6, "us", args,
                  total_dec * 1e3, {"workload": "host_step", "decode_steps_timed": steps, "threads": 1, "models": rows},
                  None, dtype="int32", higher=False)
     if ref[0] is not None:

@@ -148,13 +148,20 @@ int64_t fill_batch(MuxBatchScheduler *s, const int32_t *req, int32_t n_req,
           std::memcpy(block_tables + static_cast<int64_t>(i) * row_blocks * per, q->ids.data(),
                       sizeof(int32_t) * static_cast<size_t>(q->physical_blocks * per));
         } else {
-          // [L, n_ctx, H, row_blocks]  <-  ids[tb][l][h]
-          for (int32_t tb = 0; tb < q->physical_blocks; ++tb)
+          // [L, n_ctx, H, row_blocks]  <-  ids[tb][l][h]: a transpose of the
+          // request's [blocks][L*H] matrix, 16 token blocks at a time so that
+          // every write is one 64-byte run and the 16 source rows are each read
+          // front to back.
+          for (int32_t tb0 = 0; tb0 < q->physical_blocks; tb0 += 16) {
+            const int32_t kmax = std::min(16, q->physical_blocks - tb0);
+            const int32_t *src = q->ids.data() + static_cast<int64_t>(tb0) * per;
             for (int32_t l = 0; l < s->L; ++l) {
-              const int32_t *src = q->ids.data() + (static_cast<int64_t>(tb) * s->L + l) * s->H;
-              int32_t *dst = block_tables + ((static_cast<int64_t>(l) * n_ctx + c) * s->H) * row_blocks + tb;
-              for (int32_t h = 0; h < s->H; ++h) dst[static_cast<int64_t>(h) * row_blocks] = src[h];
+              int32_t *dst = block_tables + ((static_cast<int64_t>(l) * n_ctx + c) * s->H) * row_blocks + tb0;
+              const int32_t *sl = src + static_cast<int64_t>(l) * s->H;
+              for (int32_t h = 0; h < s->H; ++h, dst += row_blocks)
+                for (int32_t k = 0; k < kmax; ++k) dst[k] = sl[static_cast<int64_t>(k) * per + h];
             }
+          }
         }
       }
       t += 1;
