@@ -16,9 +16,13 @@
 // Packed prompts start anywhere in the token stream, so runs are not aligned
 // to multiples of 16 tokens.  The boundary between workgroups w-1 and w is
 // therefore moved back from token 16w to the start of the run that contains
-// token 16w, if there is one: both neighbours derive it from the same slots,
-// the windows still tile the token stream exactly, each holds 9..23 tokens,
-// and no run straddles two workgroups.
+// token 16w - and, when that run is the second half of a pool block whose first
+// half precedes it, on to the start of the block: inside a prompt every window
+// is then exactly one pool block (whole K and V rows, streamed past the L2),
+// whatever the prompt's position in the stream.  Both neighbours derive the
+// boundary from the same slots, the windows still tile the token stream
+// exactly, each holds 1..31 tokens, and no run straddles two workgroups.  The
+// slots are read first and only the window's own tokens are loaded.
 //
 // Fused variant (ROPE): the same kernel first applies the NeoX rotary embedding
 // to k (and to the query heads that share this kv head) for the tokens of its
@@ -83,7 +87,9 @@ __device__ __forceinline__ void store16(void *p, const uint4 x, bool streaming) 
 }
 
 constexpr int kVtRow = kHeadSize + 8;    // LDS row of one token: 256 B + 16 B so that rows shift banks
-constexpr int kSlotWin = 40;             // slots of tokens 16w-8 .. 16w+31 are examined
+constexpr int kBack = 16;                // tokens before the nominal 16 that a window may take over
+constexpr int kSlotWin = 48;             // slots of tokens 16w-16 .. 16w+31 are examined
+constexpr int kTileRows = 32;            // a window lies inside tokens 16w-16 .. 16w+15
 
 template <typename T, bool ROPE>
 __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
@@ -91,7 +97,7 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
     uint4 *__restrict__ k_pool, uint16_t *__restrict__ v_pool, int64_t num_blocks,
     const int64_t *__restrict__ slots, int64_t slot_stride, int num_tokens, int block_size, const RopeArgs R) {
   constexpr int D = kHeadSize;
-  __shared__ __attribute__((aligned(16))) uint16_t vt[24][kVtRow];
+  __shared__ __attribute__((aligned(16))) uint16_t vt[kTileRows][kVtRow];
   __shared__ int64_t s_slot[kSlotWin + 8];
   const int lane = threadIdx.x & 63;
   const int i = threadIdx.x & 15;
@@ -99,74 +105,67 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
   const int h = blockIdx.y;
   const int T0 = blockIdx.x * 16;
   const int64_t pool_slots = num_blocks * block_size;
-
-  // The nominal 16 tokens T0+i do not depend on the window: their loads go out
-  // first and overlap the slot examination.
-  const int t_nom = T0 + i;
-  const int64_t src_nom = static_cast<int64_t>(t_nom) * row_stride + h * D + c * 8;
-  uint4 kx = make_uint4(0, 0, 0, 0), vx = make_uint4(0, 0, 0, 0), kpart = make_uint4(0, 0, 0, 0);
   const int pc = (c ^ 8) - c;              // the partner chunk of the rotation, in chunks from this one
-  if (t_nom < num_tokens) {
-    kx = *reinterpret_cast<const uint4 *>(k + src_nom);
-    vx = *reinterpret_cast<const uint4 *>(v + src_nom);
-    if constexpr (ROPE) kpart = *reinterpret_cast<const uint4 *>(k + src_nom + pc * 8);
-  }
 
-  // Slots of tokens T0-8 .. T0+31; -1 for tokens outside the batch, skipped
-  // tokens and slots outside the pool (never written).
+  // Slots of tokens T0-16 .. T0+31 (bit j of the masks below is token T0-16+j);
+  // -1 for tokens outside the batch, skipped tokens and slots outside the pool
+  // (never written).
   if (threadIdx.x < kSlotWin + 8) {
-    const int t = T0 - 8 + static_cast<int>(threadIdx.x);
+    const int t = T0 - kBack + static_cast<int>(threadIdx.x);
     int64_t sl = -1;
     if (threadIdx.x < kSlotWin && t >= 0 && t < num_tokens) sl = slots[static_cast<int64_t>(t) * slot_stride + h];
     s_slot[threadIdx.x] = (sl >= 0 && sl < pool_slots) ? sl : -1;
   }
   __syncthreads();
-  // Bit j of `starts`: token T0-8+j begins a run (8 consecutive slots from a multiple of 8).
+  // Bit j of `starts`: token j begins a run (8 consecutive slots from a multiple of 8).
   bool is_start = false;
-  if (lane < 32) {
+  if (lane < 40) {
     const int64_t s0 = s_slot[lane];
     is_start = s0 >= 0 && (s0 & 7) == 0;
 #pragma unroll
     for (int e = 1; e < 8; ++e) is_start = is_start && s_slot[lane + e] == s0 + e;
   }
-  const uint32_t starts = static_cast<uint32_t>(__builtin_amdgcn_ballot_w64(is_start));
-  // Window [a, b) as bit positions [ja, jb): a run that contains a nominal
-  // boundary token belongs to the later workgroup.
-  const uint32_t before_lo = starts & 0x000000feu;        // runs starting at T0-7 .. T0-1
-  const uint32_t before_hi = starts & 0x00fe0000u;        // runs starting at T0+9 .. T0+15
-  const int ja = before_lo ? __ffs(before_lo) - 1 : 8;
-  const int jb = before_hi ? __ffs(before_hi) - 1 : min(24, num_tokens - T0 + 8);
-  const uint32_t in_win = starts & (~0u << ja) & ~(~0u << jb);   // runs that start inside the window
+  const unsigned long long starts = __builtin_amdgcn_ballot_w64(is_start);
+  // The boundary next to nominal bit n: the start of the run that contains
+  // token n, moved on to the start of that run's pool block when the run is the
+  // block's second half and the first half sits right before it - so that
+  // inside a prompt a window is exactly one pool block.  Both neighbours derive
+  // the boundary from the same slots.
+  auto boundary = [&](int n) {
+    const unsigned long long cand = starts & (0xffull << (n - 7));      // runs starting at n-7 .. n
+    if (cand == 0) return n;
+    int sbit = __ffsll(cand) - 1;
+    if (block_size == 16 && (s_slot[sbit] & 15) == 8 && ((starts >> (sbit - 8)) & 1ull) != 0 &&
+        s_slot[sbit - 8] == s_slot[sbit] - 8)
+      sbit -= 8;
+    return sbit;
+  };
+  const int ja = boundary(kBack);
+  const int jb = min(boundary(kBack + 16), num_tokens - T0 + kBack);
+  const unsigned long long in_win = starts & (~0ull << ja) & ~(~0ull << jb);   // runs that start inside the window
   // Does this window write whole pool rows and nothing else?  K rows of a run are
   // 128 bytes; a V row is block_size * 2 bytes: one run fills it at block size 8,
   // the two runs of a block at 16, never at 32.  Such a window streams its stores
   // past the L2 (uniform over the workgroup).
-  const uint32_t second = in_win & (in_win - 1);
-  const int n_runs = __popc(in_win);
+  const int n_runs = __popcll(in_win);
+  const int first_bit = n_runs > 0 ? __ffsll(in_win) - 1 : 0;
   const bool rows_complete =
       n_runs > 0 && jb - ja == 8 * n_runs &&
-      (block_size == 8 || (block_size == 16 && n_runs == 2 && __ffs(second) - __ffs(in_win) == 8 &&
-                           (s_slot[__ffs(in_win) - 1] & 15) == 0));
+      (block_size == 8 || (block_size == 16 && n_runs == 2 && ((in_win >> (first_bit + 8)) & 1ull) != 0 &&
+                           (s_slot[first_bit] & 15) == 0 && s_slot[first_bit + 8] == s_slot[first_bit] + 8));
 
-  // Rows of the LDS tile are bit positions: 8 + i for the nominal tokens, i for
-  // the up to 7 tokens taken over from the previous workgroup's nominal range.
+  // Rows of the LDS tile are bit positions: 16 + i for the nominal tokens, i for
+  // the up to 15 tokens taken over from the previous workgroup's nominal range.
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
-    const int j = pass == 0 ? 8 + i : i;
-    const bool mine = j >= ja && j < jb && (pass == 0 || i < 8);     // token T0-8+j is in this window
-    const int t = T0 - 8 + j;
+    if (pass == 1 && ja == kBack) break;   // uniform: no token taken over from the previous workgroup
+    const int j = pass == 0 ? kBack + i : i;
+    const bool mine = j >= ja && j < jb;                   // token T0-16+j is in this window
+    const int t = T0 - kBack + j;
     const int64_t src = static_cast<int64_t>(t) * row_stride + h * D + c * 8;
-    if (pass == 1) {
-      if (ja == 8) break;                // uniform: no token taken over from the previous workgroup
-      if constexpr (!ROPE) {
-        if (i >= 8) break;
-      }
-      kx = make_uint4(0, 0, 0, 0);
-      vx = make_uint4(0, 0, 0, 0);
-      kpart = make_uint4(0, 0, 0, 0);
-    }
     const int64_t slot = mine ? s_slot[j] : -1;
-    if (pass == 1 && mine && (ROPE || slot >= 0)) {
+    uint4 kx = make_uint4(0, 0, 0, 0), vx = make_uint4(0, 0, 0, 0), kpart = make_uint4(0, 0, 0, 0);
+    if (mine && (ROPE || slot >= 0)) {
       kx = *reinterpret_cast<const uint4 *>(k + src);
       vx = *reinterpret_cast<const uint4 *>(v + src);
       if constexpr (ROPE) kpart = *reinterpret_cast<const uint4 *>(k + src + pc * 8);
@@ -210,7 +209,7 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
       const int64_t blk = slot / block_size;
       const int o = static_cast<int>(slot - blk * block_size);
       // Element path for tokens that no run covers (a run starts at most 7 tokens back).
-      const uint32_t cover = in_win & (0xffu << (j > 7 ? j - 7 : 0)) & ~(~0u << (j + 1));
+      const unsigned long long cover = in_win & (0xffull << (j > 7 ? j - 7 : 0)) & ~(~0ull << (j + 1));
       store16(&k_pool[(blk * (D / 8) + c) * block_size + o], kx, rows_complete);
       if (cover == 0) {
         uint16_t *vp = v_pool + (blk * D + c * 8) * block_size + o;
@@ -222,15 +221,15 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
         }
       }
     }
-    if (in_win != 0 && (pass == 0 || i < 8)) *reinterpret_cast<uint4 *>(&vt[j][c * 8]) = vx;
+    if (in_win != 0) *reinterpret_cast<uint4 *>(&vt[j][c * 8]) = vx;
   }
   if (in_win == 0) return;                                 // uniform: no run in this window
   __syncthreads();
-  // Up to two runs per window; thread (c, i) stores dim 8c + i%8 of run i/8.
-  uint32_t m = in_win;
-  if (i >= 8) m &= m - 1;                                  // drop the first run
-  if (m != 0) {
-    const int jp = __ffs(m) - 1;                           // bit, and LDS row, of the run's first token
+  // Up to three runs per window; thread (c, i) stores dim 8c + i%8 of runs i/8, i/8 + 2.
+  for (int r = i >> 3; r < n_runs; r += 2) {
+    unsigned long long m = in_win;
+    for (int q = 0; q < r; ++q) m &= m - 1;                // drop the runs before run r
+    const int jp = __ffsll(m) - 1;                         // bit, and LDS row, of the run's first token
     const int d = c * 8 + (i & 7);
     uint32_t w[4];
 #pragma unroll
