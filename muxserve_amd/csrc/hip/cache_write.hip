@@ -77,10 +77,12 @@ __device__ __forceinline__ void store16(void *p, const uint4 x, bool streaming) 
   const cw_u32x4 v = {x.x, x.y, x.z, x.w};
   if (streaming) {
     // Written as an instruction: as two C++ stores that differ only in the hint,
-    // the optimiser folds the branches into one store and drops it.  The s_nop
-    // covers the wait state between a 16-byte store and a write of its data
-    // registers.
-    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 0" ::"v"(p), "v"(v) : "memory");
+    // the optimiser folds the branches into one store and drops it.  The
+    // compiler does not know that the instruction is still reading its data
+    // registers when the next one issues, so the wait states between a 16-byte
+    // store and a write of its data registers are spelled out (one was not
+    // enough once the next store's operands were already in registers).
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 4" ::"v"(p), "v"(v) : "memory");
   } else {
     *static_cast<cw_u32x4 *>(p) = v;
   }
@@ -102,8 +104,11 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
   const int lane = threadIdx.x & 63;
   const int i = threadIdx.x & 15;
   const int c = threadIdx.x >> 4;
-  const int h = blockIdx.y;
-  const int T0 = blockIdx.x * 16;
+  // Heads vary fastest over the workgroup ids: workgroups that run together read
+  // the neighbouring 256-byte head slices of the same k/v rows (one DRAM page)
+  // rather than one slice out of each of many rows.
+  const int h = blockIdx.x;
+  const int T0 = blockIdx.y * 16;
   const int64_t pool_slots = num_blocks * block_size;
   const int pc = (c ^ 8) - c;              // the partner chunk of the rotation, in chunks from this one
 
@@ -154,22 +159,36 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
       (block_size == 8 || (block_size == 16 && n_runs == 2 && ((in_win >> (first_bit + 8)) & 1ull) != 0 &&
                            (s_slot[first_bit] & 15) == 0 && s_slot[first_bit + 8] == s_slot[first_bit] + 8));
 
-  // Rows of the LDS tile are bit positions: 16 + i for the nominal tokens, i for
-  // the up to 15 tokens taken over from the previous workgroup's nominal range.
+  // Thread (c, i) takes the window's tokens ja + i and, in the rare window of
+  // more than 16 tokens, ja + 16 + i: inside a prompt the 16 threads of a chunk
+  // row then write one whole 256-byte K row with a single store instruction
+  // (split over two instructions, the non-temporal stores would each leave
+  // partial lines).  Rows of the LDS tile are bit positions.  Both passes' loads
+  // go out before anything is stored.
+  const bool two_passes = jb - ja > 16;                    // uniform
+  uint4 kx2[2], vx2[2], kp2[2];
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
-    if (pass == 1 && ja == kBack) break;   // uniform: no token taken over from the previous workgroup
-    const int j = pass == 0 ? kBack + i : i;
-    const bool mine = j >= ja && j < jb;                   // token T0-16+j is in this window
+    kx2[pass] = vx2[pass] = kp2[pass] = make_uint4(0, 0, 0, 0);
+    if (pass == 1 && !two_passes) break;
+    const int j = ja + 16 * pass + i;
+    if (j < jb && (ROPE || s_slot[j] >= 0)) {
+      const int64_t src = static_cast<int64_t>(T0 - kBack + j) * row_stride + h * D + c * 8;
+      kx2[pass] = *reinterpret_cast<const uint4 *>(k + src);
+      vx2[pass] = *reinterpret_cast<const uint4 *>(v + src);
+      if constexpr (ROPE) kp2[pass] = *reinterpret_cast<const uint4 *>(k + src + pc * 8);
+    }
+  }
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    if (pass == 1 && !two_passes) break;
+    const int j = ja + 16 * pass + i;
+    const bool mine = j < jb;                              // token T0-16+j is in this window
     const int t = T0 - kBack + j;
     const int64_t src = static_cast<int64_t>(t) * row_stride + h * D + c * 8;
     const int64_t slot = mine ? s_slot[j] : -1;
-    uint4 kx = make_uint4(0, 0, 0, 0), vx = make_uint4(0, 0, 0, 0), kpart = make_uint4(0, 0, 0, 0);
-    if (mine && (ROPE || slot >= 0)) {
-      kx = *reinterpret_cast<const uint4 *>(k + src);
-      vx = *reinterpret_cast<const uint4 *>(v + src);
-      if constexpr (ROPE) kpart = *reinterpret_cast<const uint4 *>(k + src + pc * 8);
-    }
+    uint4 kx = kx2[pass];
+    const uint4 vx = vx2[pass], kpart = kp2[pass];
     if constexpr (ROPE) {
       // Rotate k of every token of the window (also tokens without a slot), and
       // the query heads of this kv head, four at a time; all reads of a group
@@ -221,7 +240,7 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
         }
       }
     }
-    if (in_win != 0) *reinterpret_cast<uint4 *>(&vt[j][c * 8]) = vx;
+    if (in_win != 0 && mine) *reinterpret_cast<uint4 *>(&vt[j][c * 8]) = vx;
   }
   if (in_win == 0) return;                                 // uniform: no run in this window
   __syncthreads();
@@ -262,7 +281,7 @@ int32_t check_cache_write(const void *k, const void *v, int64_t kv_row_stride, c
   const uintptr_t align = reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
                           reinterpret_cast<uintptr_t>(k_pool) | reinterpret_cast<uintptr_t>(v_pool);
   if (align & 15u) return MUXA_EINVAL;
-  if (num_kv_heads > 65535) return MUXA_EUNSUPPORTED;
+  if (num_tokens > 16 * 65535) return MUXA_EUNSUPPORTED;      // one grid row per 16 tokens
   if (num_pool_blocks > (int64_t{1} << 56)) return MUXA_EINVAL;   // slot arithmetic stays in 64 bits
   return MUXA_OK;
 }
@@ -282,7 +301,7 @@ extern "C" int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t k
   if (num_tokens == 0) return MUXA_OK;
   const int64_t slot_stride = static_cast<int64_t>(num_layers) * num_kv_heads;
   const int64_t *slots = slot_mapping + static_cast<int64_t>(layer) * num_kv_heads;
-  dim3 grid((num_tokens + 15) / 16, num_kv_heads);
+  dim3 grid(num_kv_heads, (num_tokens + 15) / 16);
   // Without the rotary part the kernel only moves bytes and never writes k.
   hipLaunchKernelGGL((reshape_and_cache_kernel<F16, false>), grid, dim3(256), 0, static_cast<hipStream_t>(stream),
                      const_cast<uint16_t *>(static_cast<const uint16_t *>(k)), static_cast<const uint16_t *>(v),
@@ -321,7 +340,7 @@ extern "C" int32_t mux_rope_reshape_and_cache(const int64_t *positions, void *q,
   R.positions = positions;
   R.cos_sin = cos_sin;
   R.max_position = max_position;
-  dim3 grid((num_tokens + 15) / 16, num_kv_heads);
+  dim3 grid(num_kv_heads, (num_tokens + 15) / 16);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == MUXA_DTYPE_F16)
     hipLaunchKernelGGL((reshape_and_cache_kernel<F16, true>), grid, dim3(256), 0, st, static_cast<uint16_t *>(k),
