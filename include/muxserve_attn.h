@@ -212,7 +212,7 @@ int32_t mux_silu_and_mul(void *out, int64_t out_row_stride, const void *x, int64
 
 /* mux_greedy_sample: GreedySampler.forward (sampler.py:15-35) without
  * materialising the logits.  For sampled row r < num_rows:
- *     h = hidden_states[row_index ? row_index[r] : r]
+ *     h = hidden_states[row_index ? row_index[r] : r]     (entries clamped to num_hidden_rows - 1)
  *     next_tokens[r] = argmax_{v < vocab_size} T(h . embedding[v,:])
  * (fp32 accumulation, each logit rounded to T before the comparison as the
  * reference's fp16 logits are; ties go to the lowest id).  On a prompt step
@@ -229,7 +229,8 @@ int32_t mux_silu_and_mul(void *out, int64_t out_row_stride, const void *x, int64
 size_t mux_greedy_sample_workspace_bytes(int32_t vocab_size);
 int32_t mux_greedy_sample_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
 int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_states, int64_t hidden_row_stride,
-                          const int32_t *row_index, int32_t num_rows, const void *embedding,
+                          int32_t num_hidden_rows, const int32_t *row_index, int32_t num_rows,
+                          const void *embedding,
                           int64_t embedding_row_stride, int32_t embedding_rows, int32_t vocab_size,
                           int32_t hidden_size, int32_t dtype, void *workspace, size_t workspace_bytes,
                           void *stream);

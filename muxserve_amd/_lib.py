@@ -136,7 +136,7 @@ ATTN_SIGNATURES = {
     "mux_silu_and_mul": (c_i32, [c_vp, c_i64, c_vp, c_i64, c_i32, c_i32, c_i32, c_vp]),
     "mux_greedy_sample_workspace_bytes": (c_sz, [c_i32]),
     "mux_greedy_sample_workspace_init": (c_i32, [c_vp, c_sz, c_vp]),
-    "mux_greedy_sample": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_i32, c_vp, c_i64, c_i32, c_i32, c_i32, c_i32,
+    "mux_greedy_sample": (c_i32, [c_vp, c_vp, c_i64, c_i32, c_vp, c_i32, c_vp, c_i64, c_i32, c_i32, c_i32, c_i32,
                                   c_vp, c_sz, c_vp]),
     "mux_build_step_inputs": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_i32, c_vp, c_i64, c_i32,
                                       c_i32, c_vp, c_vp, c_i32, c_vp]),

@@ -111,7 +111,9 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
   if (group >= P.num_groups) return;
   const int in_group = slot % per_group;
   const int prompt_rank = group / P.num_kv_heads;
-  const int prompt = P.prompt_order ? P.prompt_order[prompt_rank] : prompt_rank;
+  // (an entry outside the batch is clamped: a malformed order costs results, never a stray read)
+  const int prompt =
+      P.prompt_order ? min(max(P.prompt_order[prompt_rank], 0), P.num_groups / P.num_kv_heads - 1) : prompt_rank;
   const int hk = group % P.num_kv_heads;
   const int hq = hk * P.ratio + in_group / P.q_tiles;
   const int seq_begin = P.cu_seqlens[prompt];

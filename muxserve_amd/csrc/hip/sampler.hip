@@ -55,6 +55,7 @@ struct LmHeadParams {
   const uint16_t *weight;
   int64_t weight_stride;
   int32_t hidden_size, vocab, num_rows;
+  int32_t hidden_rows;                    // rows of `hidden`: row_index entries are clamped to it
   uint32_t *counter;                      // workgroups arrived, zero between launches
   unsigned long long *table;              // [workgroups][16 NB] keys, written before they are read
   int64_t *next_tokens;
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadPar
     const int row = (tid >> 4) + RPP * j;
     hstore[j] = row < ROWS;
     hvalid[j] = row < P.num_rows && hstore[j];
-    const int src = hvalid[j] ? (P.row_index ? P.row_index[row] : row) : 0;
+    const int src = hvalid[j] ? (P.row_index ? min(max(P.row_index[row], 0), P.hidden_rows - 1) : row) : 0;
     hsrc[j] = P.hidden + static_cast<int64_t>(src) * P.hidden_stride + 8 * (tid & 15);
   }
   const int hoff = (tid >> 4) * kHRow + 8 * (tid & 15);
@@ -334,13 +335,15 @@ extern "C" int32_t mux_greedy_sample_workspace_init(void *workspace, size_t work
 }
 
 extern "C" int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_states, int64_t hidden_row_stride,
-                                     const int32_t *row_index, int32_t num_rows, const void *embedding,
+                                     int32_t num_hidden_rows, const int32_t *row_index, int32_t num_rows,
+                                     const void *embedding,
                                      int64_t embedding_row_stride, int32_t embedding_rows, int32_t vocab_size,
                                      int32_t hidden_size, int32_t dtype, void *workspace, size_t workspace_bytes,
                                      void *stream) {
   using namespace mux;
   if (!next_tokens || !hidden_states || !embedding) return MUXA_EINVAL;
   if (num_rows < 0 || vocab_size <= 0 || hidden_size <= 0 || embedding_rows < vocab_size) return MUXA_EINVAL;
+  if (num_hidden_rows < 1 || (!row_index && num_rows > num_hidden_rows)) return MUXA_EINVAL;
   if (dtype != MUXA_DTYPE_F16 && dtype != MUXA_DTYPE_BF16) return MUXA_EUNSUPPORTED;
   if (hidden_size % kSmTile) return MUXA_EUNSUPPORTED;
   if (hidden_row_stride < hidden_size || embedding_row_stride < hidden_size || hidden_row_stride % 8 ||
@@ -373,6 +376,7 @@ extern "C" int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_st
     P.hidden_size = hidden_size;
     P.vocab = vocab_size;
     P.num_rows = rows;
+    P.hidden_rows = row_index ? num_hidden_rows : num_hidden_rows - r0;
     P.counter = static_cast<uint32_t *>(workspace);
     P.table = reinterpret_cast<unsigned long long *>(static_cast<char *>(workspace) + kSmCounterBytes);
     P.next_tokens = next_tokens + r0;

@@ -329,8 +329,9 @@ def greedy_sample(embedding: torch.Tensor, hidden_states: torch.Tensor, vocab_si
         if workspace is None or workspace.numel() < need:
             workspace = torch.zeros(max(need, 1), dtype=torch.uint8, device=hidden_states.device)   # born zeroed
             _sample_workspaces[key] = workspace
-    rc = lib.mux_greedy_sample(out.data_ptr(), hidden_states.data_ptr(), _rows(hidden_states, "hidden_states"), ri_ptr,
-                               num_rows, embedding.data_ptr(), _rows(embedding, "embedding"), embedding.shape[0],
+    rc = lib.mux_greedy_sample(out.data_ptr(), hidden_states.data_ptr(), _rows(hidden_states, "hidden_states"),
+                               hidden_states.shape[0], ri_ptr, num_rows, embedding.data_ptr(),
+                               _rows(embedding, "embedding"), embedding.shape[0],
                                int(vocab_size), hidden_states.shape[1], _dtype_code(hidden_states),
                                workspace.data_ptr(), workspace.numel(), _stream_ptr(stream))
     _lib.check_attn(rc, "mux_greedy_sample")
