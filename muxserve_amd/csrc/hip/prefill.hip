@@ -235,6 +235,14 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
     }
   };
 
+  // Lane-dependent part of the V^T fragment addresses (see read_v), in elements.
+  int v_lane_base[2];
+  {
+    const int jrow = (lane & 15) >> 2, m = lane & 3;
+    const int rl = 4 * half + jrow, cl = 2 * ((lane >> 4) & 1) + (m >> 1);
+    v_lane_base[0] = rl * D + 8 * (cl ^ rl) + 4 * (m & 1);
+    v_lane_base[1] = rl * D + 8 * (cl ^ rl ^ 4) + 4 * (m & 1);
+  }
   if constexpr (DMA) dma_tile(0);
   else load_tile();
   for (int t = 0; t < n_tiles; ++t) {
@@ -371,14 +379,16 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
           // group points at dims 4 m .. 4 m + 3 of key row j, and lane i of the
           // group receives dim i of rows 0..3.  Here a group covers dims
           // 32 mb + 16 (lane/16 % 2) .. +15 and keys 16 ks + 4 half (+ 8) .. +3.
+          // Address: row = 16 ks + 8 hsel + rl with rl = 4 half + jrow, chunk =
+          // 4 mb + cl, position = chunk ^ (row % 16) = (cl ^ rl) ^ 4 (mb ^ 2 hsel).
+          // The lane part cl ^ rl is below 8, so bit 3 of the constant part adds
+          // and only its bit 2 (mb odd) has to be folded into the lane's base:
+          // two bases per lane, everything else is an immediate offset.
           typedef __attribute__((address_space(3))) v4i16 lds_v4i16;
-          const int jrow = (lane & 15) >> 2, m = lane & 3;
-          const int chunk = 4 * mb + 2 * ((lane >> 4) & 1) + (m >> 1);
           u32x2 part[2];
 #pragma unroll
           for (int hsel = 0; hsel < 2; ++hsel) {
-            const int row = 16 * ks + 8 * hsel + 4 * half + jrow;
-            const uint16_t *src = Vr + row * D + 8 * (chunk ^ (row & 15)) + 4 * (m & 1);
+            const uint16_t *src = Vr + v_lane_base[mb & 1] + (16 * ks + 8 * hsel) * D + 64 * (((mb >> 1) ^ hsel) & 1);
             const v4i16 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16 *)src);
             union { v4i16 v; u32x2 u; } c;
             c.v = r;
