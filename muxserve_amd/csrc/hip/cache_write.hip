@@ -1,16 +1,18 @@
 // KV-cache write (reshape_and_cache) into the head-granular pool, gfx950.
 //
 // Pure byte movement.  A 256-thread workgroup takes about 16 consecutive
-// tokens of one kv head; thread (c, i) loads the 16-byte chunk c (dims
-// 8c..8c+7) of token i of both K and V:
+// tokens of one kv head.  Loading, thread (i, c) takes the 16-byte chunk c (dims
+// 8c..8c+7) of token i of both K and V, so that a token's 256-byte head slice is
+// read by 16 neighbouring threads; the tile goes to LDS, one row per token, and
+// is stored from there by thread (c, i):
 //   K pool [D/8][BS][8]: the chunk goes out as one 16-byte store; the token
 //     lanes of a chunk row are adjacent, so tokens in consecutive slots of one
 //     block fill a contiguous run.
 //   V pool [D][BS]: 8 consecutive tokens of one dim are a 16-byte chunk of the
 //     pool.  Where 8 consecutive tokens go to 8 consecutive slots that start at
 //     a multiple of 8 (every prompt written through a block table does, up to
-//     its last few tokens) the tile is transposed through LDS and one thread
-//     stores the whole chunk of a dim.  Tokens outside such runs (decode steps,
+//     its last few tokens) one thread gathers a dim's 8 values from the LDS rows
+//     and stores the whole chunk.  Tokens outside such runs (decode steps,
 //     arbitrary slots, prompt tails) take the element path: a chunk's 8 dims
 //     as 8 two-byte stores BS*2 bytes apart.
 // Packed prompts start anywhere in the token stream, so runs are not aligned
@@ -99,6 +101,7 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
     uint4 *__restrict__ k_pool, uint16_t *__restrict__ v_pool, int64_t num_blocks,
     const int64_t *__restrict__ slots, int64_t slot_stride, int num_tokens, int block_size, const RopeArgs R) {
   constexpr int D = kHeadSize;
+  __shared__ __attribute__((aligned(16))) uint16_t kt[kTileRows][kVtRow];
   __shared__ __attribute__((aligned(16))) uint16_t vt[kTileRows][kVtRow];
   __shared__ int64_t s_slot[kSlotWin + 8];
   const int lane = threadIdx.x & 63;
@@ -110,7 +113,6 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
   const int h = blockIdx.x;
   const int T0 = blockIdx.y * 16;
   const int64_t pool_slots = num_blocks * block_size;
-  const int pc = (c ^ 8) - c;              // the partner chunk of the rotation, in chunks from this one
 
   // Slots of tokens T0-16 .. T0+31 (bit j of the masks below is token T0-16+j);
   // -1 for tokens outside the batch, skipped tokens and slots outside the pool
@@ -159,21 +161,28 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
       (block_size == 8 || (block_size == 16 && n_runs == 2 && ((in_win >> (first_bit + 8)) & 1ull) != 0 &&
                            (s_slot[first_bit] & 15) == 0 && s_slot[first_bit + 8] == s_slot[first_bit] + 8));
 
-  // Thread (c, i) takes the window's tokens ja + i and, in the rare window of
-  // more than 16 tokens, ja + 16 + i: inside a prompt the 16 threads of a chunk
-  // row then write one whole 256-byte K row with a single store instruction
-  // (split over two instructions, the non-temporal stores would each leave
-  // partial lines).  Rows of the LDS tile are bit positions.  Both passes' loads
-  // go out before anything is stored.
+  // Loads: thread (token il, chunk cl) - the 16 threads of a token read its whole
+  // 256-byte head slice, a wave four such slices, every line exactly once.
+  // (Non-temporal loads make no difference whether k/v come from HBM or were
+  // just written by the projection, and lose when the same buffers are read
+  // again.)  Stores: thread
+  // (chunk row c, token i) - the 16 threads of a chunk row write one whole
+  // 256-byte K row of the block with a single store instruction (split over
+  // two, the non-temporal stores would each leave partial lines).  In between
+  // the tile sits in LDS, one row per token (rows are bit positions); V is
+  // transposed on its way out.  A window has at most 31 tokens: two passes of
+  // 16, the second one rare.
   const bool two_passes = jb - ja > 16;                    // uniform
+  const int il = threadIdx.x >> 4, cl = threadIdx.x & 15;
+  const int pc = (cl ^ 8) - cl;            // the partner chunk of the rotation, in chunks from this one
   uint4 kx2[2], vx2[2], kp2[2];
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
     kx2[pass] = vx2[pass] = kp2[pass] = make_uint4(0, 0, 0, 0);
     if (pass == 1 && !two_passes) break;
-    const int j = ja + 16 * pass + i;
+    const int j = ja + 16 * pass + il;
     if (j < jb && (ROPE || s_slot[j] >= 0)) {
-      const int64_t src = static_cast<int64_t>(T0 - kBack + j) * row_stride + h * D + c * 8;
+      const int64_t src = static_cast<int64_t>(T0 - kBack + j) * row_stride + h * D + cl * 8;
       kx2[pass] = *reinterpret_cast<const uint4 *>(k + src);
       vx2[pass] = *reinterpret_cast<const uint4 *>(v + src);
       if constexpr (ROPE) kp2[pass] = *reinterpret_cast<const uint4 *>(k + src + pc * 8);
@@ -182,32 +191,30 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
     if (pass == 1 && !two_passes) break;
-    const int j = ja + 16 * pass + i;
+    const int j = ja + 16 * pass + il;
     const bool mine = j < jb;                              // token T0-16+j is in this window
-    const int t = T0 - kBack + j;
-    const int64_t src = static_cast<int64_t>(t) * row_stride + h * D + c * 8;
-    const int64_t slot = mine ? s_slot[j] : -1;
     uint4 kx = kx2[pass];
-    const uint4 vx = vx2[pass], kpart = kp2[pass];
     if constexpr (ROPE) {
       // Rotate k of every token of the window (also tokens without a slot), and
       // the query heads of this kv head, four at a time; all reads of a group
       // precede its writes (the workgroup meets in between), because a thread's
       // partner chunk is another thread's own.
+      const int t = T0 - kBack + j;
+      const int64_t src = static_cast<int64_t>(t) * row_stride + h * D + cl * 8;
       float cs[8], sn[8];
       if (mine) {
         int64_t pos = R.positions[t];
         pos = pos < 0 ? 0 : (pos >= R.max_position ? R.max_position - 1 : pos);
-        const float *row = R.cos_sin + pos * D + (c & 7) * 8;
+        const float *row = R.cos_sin + pos * D + (cl & 7) * 8;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           cs[e] = row[e];
           sn[e] = row[D / 2 + e];
         }
-        kx = rotate_chunk<T>(kx, kpart, cs, sn, c >= 8);
+        kx = rotate_chunk<T>(kx, kp2[pass], cs, sn, cl >= 8);
       }
       const int n_q = R.q != nullptr ? R.ratio : 0;
-      uint16_t *q0 = R.q + static_cast<int64_t>(t) * R.q_stride + static_cast<int64_t>(h) * R.ratio * D + c * 8;
+      uint16_t *q0 = R.q + static_cast<int64_t>(t) * R.q_stride + static_cast<int64_t>(h) * R.ratio * D + cl * 8;
       for (int g0 = 0; g0 < max(n_q, 1); g0 += 4) {
         uint4 qx[4];
 #pragma unroll
@@ -215,7 +222,7 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
           if (mine && g0 + g < n_q) {
             const uint16_t *qp = q0 + (g0 + g) * D;
             qx[g] = rotate_chunk<T>(*reinterpret_cast<const uint4 *>(qp),
-                                    *reinterpret_cast<const uint4 *>(qp + pc * 8), cs, sn, c >= 8);
+                                    *reinterpret_cast<const uint4 *>(qp + pc * 8), cs, sn, cl >= 8);
           }
         __syncthreads();
         if (mine && g0 == 0) *reinterpret_cast<uint4 *>(k + src) = kx;
@@ -224,14 +231,27 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
           if (mine && g0 + g < n_q) *reinterpret_cast<uint4 *>(q0 + (g0 + g) * D) = qx[g];
       }
     }
+    if (mine) {
+      *reinterpret_cast<uint4 *>(&kt[j][cl * 8]) = kx;
+      *reinterpret_cast<uint4 *>(&vt[j][cl * 8]) = vx2[pass];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    if (pass == 1 && !two_passes) break;
+    const int j = ja + 16 * pass + i;
+    const int64_t slot = j < jb ? s_slot[j] : -1;
     if (slot >= 0) {
       const int64_t blk = slot / block_size;
       const int o = static_cast<int>(slot - blk * block_size);
       // Element path for tokens that no run covers (a run starts at most 7 tokens back).
       const unsigned long long cover = in_win & (0xffull << (j > 7 ? j - 7 : 0)) & ~(~0ull << (j + 1));
-      store16(&k_pool[(blk * (D / 8) + c) * block_size + o], kx, rows_complete);
+      store16(&k_pool[(blk * (D / 8) + c) * block_size + o], *reinterpret_cast<const uint4 *>(&kt[j][c * 8]),
+              rows_complete);
       if (cover == 0) {
         uint16_t *vp = v_pool + (blk * D + c * 8) * block_size + o;
+        const uint4 vx = *reinterpret_cast<const uint4 *>(&vt[j][c * 8]);
         const uint32_t w[4] = {vx.x, vx.y, vx.z, vx.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -240,10 +260,7 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
         }
       }
     }
-    if (in_win != 0 && mine) *reinterpret_cast<uint4 *>(&vt[j][c * 8]) = vx;
   }
-  if (in_win == 0) return;                                 // uniform: no run in this window
-  __syncthreads();
   // Up to three runs per window; thread (c, i) stores dim 8c + i%8 of runs i/8, i/8 + 2.
   for (int r = i >> 3; r < n_runs; r += 2) {
     unsigned long long m = in_win;
