@@ -46,6 +46,7 @@ class InputMetadata:
     is_muxserve: bool = True                   # read at models/llama.py:285
     _cu_seqlens: Optional[torch.Tensor] = field(default=None, repr=False)
     _prompt_order: Optional[torch.Tensor] = field(default=None, repr=False)
+    _last_rows: Optional[torch.Tensor] = field(default=None, repr=False)
 
     def __post_init__(self):
         self.prompt_lens = [int(x) for x in self.prompt_lens]
@@ -66,6 +67,17 @@ class InputMetadata:
                 cu.append(cu[-1] + n)
             self._cu_seqlens = torch.tensor(cu, dtype=torch.int32, device=device)
         return self._cu_seqlens
+
+    def last_token_rows(self, device) -> torch.Tensor:
+        """int32 [num_prompts] on the device: the row of every prompt's last token
+        (cumsum(prompt_lens) - 1, what the sampler looks at), built once per step."""
+        if self._last_rows is None or self._last_rows.device != torch.device(device):
+            rows, end = [], 0
+            for n in self.prompt_lens:
+                end += n
+                rows.append(end - 1)
+            self._last_rows = torch.tensor(rows, dtype=torch.int32, device=device)
+        return self._last_rows
 
     def prompt_order(self, device) -> torch.Tensor:
         """int32 [num_prompts] on the device: the prompts longest first (the order

@@ -46,8 +46,11 @@ class GreedySampler(torch.nn.Module):
         row_index = None
         if input_metadata.num_prompts > 0:
             assert input_metadata.num_generation_tokens == 0           # sampler.py:19
-            indices = np.cumsum(input_metadata.prompt_lens) - 1         # sampler.py:20
-            row_index = torch.tensor(indices, dtype=torch.int32, device=hidden_states.device)
+            if hasattr(input_metadata, "last_token_rows"):              # cached per step by this package's metadata
+                row_index = input_metadata.last_token_rows(hidden_states.device)
+            else:
+                indices = np.cumsum(input_metadata.prompt_lens) - 1     # sampler.py:20
+                row_index = torch.tensor(indices, dtype=torch.int32, device=hidden_states.device)
             num_tokens = input_metadata.num_prompts
         else:
             num_tokens = input_metadata.num_generation_tokens
