@@ -433,3 +433,43 @@ def test_decode_config2_full_size_pool():
     for m, t in zip(models, tables):
         want = orc.paged_decode(m.q.cpu(), ks, vs, t, m.context_lens, m.scale)
         _check(m.out[:m.batch].float().cpu(), want)
+
+
+@pytest.mark.parametrize("Hq,Hkv,dtype", [(4, 4, torch.float16), (16, 2, torch.bfloat16)])
+def test_decode_is_invariant_under_relabelling_of_the_physical_blocks(Hq, Hkv, dtype):
+    """The same logical caches stored under different block ids (pool permuted,
+    tables relabelled) give bit-identical outputs: nothing in the result may
+    depend on where a block lives.  Contexts cover single-partition, split and
+    remainder units; the write goes through the GPU cache-write kernel."""
+    print(f"[case] decode block relabelling Hq={Hq} Hkv={Hkv} {dtype}", flush=True)
+    bs = 16
+    rng = np.random.Generator(np.random.PCG64(31))
+    g = torch.Generator().manual_seed(31)
+    ctx = np.asarray([1, 16, 70, 256, 257, 700, 1300, 33], dtype=np.int32)
+    B = len(ctx)
+    nblk = (ctx.astype(np.int64) + bs - 1) // bs
+    need = int(nblk.sum()) * Hkv
+    N = 3 * need + 11
+    pad = (B + 7) // 8 * 8
+    q = torch.randn((pad, Hq * HEAD_SIZE), generator=g).to(dtype).to(DEV)
+    dense = [(torch.randn((int(n), Hkv * HEAD_SIZE), generator=g).to(dtype),
+              torch.randn((int(n), Hkv * HEAD_SIZE), generator=g).to(dtype)) for n in ctx]
+    outs = []
+    for trial in range(3):
+        ids = rng.permutation(N)[:need]
+        bt1, _ = workloads.build_tables(ctx, Hkv, bs, ids)
+        k_pool, v_pool = allocate_gpu_cache(N, bs, DEV, dtype=dtype)
+        k_pool.fill_(float("nan"))
+        v_pool.fill_(float("nan"))
+        for s_, (kd, vd) in enumerate(dense):
+            n = int(ctx[s_])
+            i = np.arange(n)
+            slots = bt1[0, s_][:, i // bs].astype(np.int64).T * bs + (i % bs)[:, None]
+            ops.reshape_and_cache(kd.to(DEV), vd.to(DEV), k_pool, v_pool,
+                                  torch.from_numpy(np.ascontiguousarray(slots[:, None, :])).to(DEV))
+        out = torch.zeros((pad, Hq * HEAD_SIZE), dtype=dtype, device=DEV)
+        ops.paged_decode(out, q, k_pool, v_pool, torch.from_numpy(bt1).to(DEV), torch.from_numpy(ctx).to(DEV),
+                         int(ctx.max()), HEAD_SIZE ** -0.5)
+        torch.cuda.synchronize()
+        outs.append(out[:B].cpu().view(torch.int16))
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
