@@ -128,17 +128,25 @@ class DecodeCall:
 _workspaces = {}
 
 
-def _workspace(nbytes: int, device) -> Optional[torch.Tensor]:
-    """Grow-only scratch for split partials, one per (device, stream).  Born
-    zeroed: it starts with arrival counters that every launch leaves at zero."""
+def _scratch(cache: dict, nbytes: int, device, stream_ptr: int, floor: int) -> Optional[torch.Tensor]:
+    """Grow-only zero-filled scratch, one per (device, stream the launch goes
+    to).  The fill runs on torch's current stream, which need not be that
+    stream, so a new buffer is waited for once before its first use."""
     if nbytes == 0:
         return None
-    key = (device, torch.cuda.current_stream(device).cuda_stream)
-    ws = _workspaces.get(key)
+    key = (device, stream_ptr)
+    ws = cache.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
+        ws = torch.zeros(max(nbytes, floor), dtype=torch.uint8, device=device)
+        torch.cuda.current_stream(device).synchronize()
+        cache[key] = ws
     return ws
+
+
+def _workspace(nbytes: int, device, stream_ptr: int) -> Optional[torch.Tensor]:
+    """Scratch for split partials.  Born zeroed: it starts with arrival counters
+    that every launch leaves at zero."""
+    return _scratch(_workspaces, nbytes, device, stream_ptr, 1 << 20)
 
 
 def multi_decode(calls: List[DecodeCall], k_pool: torch.Tensor, v_pool: torch.Tensor,
@@ -154,11 +162,12 @@ def multi_decode(calls: List[DecodeCall], k_pool: torch.Tensor, v_pool: torch.Te
             raise TypeError("q dtype must equal the pool dtype")
     lib = _lib.attn()
     need = lib.mux_paged_decode_workspace_bytes(ctypes.addressof(items), len(calls), int(partition_size))
-    ws = workspace if workspace is not None else _workspace(need, k_pool.device)
+    sp = _stream_ptr(stream)
+    ws = workspace if workspace is not None else _workspace(need, k_pool.device, sp)
     ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)
     rc = lib.mux_multi_decode(ctypes.addressof(items), len(calls), k_pool.data_ptr(), v_pool.data_ptr(),
                               k_pool.shape[0], HEAD_SIZE, bs, _dtype_code(k_pool), int(partition_size),
-                              ws_ptr, ws_bytes, _stream_ptr(stream))
+                              ws_ptr, ws_bytes, sp)
     _lib.check_attn(rc, "mux_multi_decode")
 
 
@@ -323,17 +332,14 @@ def greedy_sample(embedding: torch.Tensor, hidden_states: torch.Tensor, vocab_si
         raise ValueError("out: expected contiguous int64 [>= num_rows]")
     lib = _lib.attn()
     need = lib.mux_greedy_sample_workspace_bytes(int(vocab_size))
+    sp = _stream_ptr(stream)
     if workspace is None:
-        key = (hidden_states.device, torch.cuda.current_stream(hidden_states.device).cuda_stream)
-        workspace = _sample_workspaces.get(key)
-        if workspace is None or workspace.numel() < need:
-            workspace = torch.zeros(max(need, 1), dtype=torch.uint8, device=hidden_states.device)   # born zeroed
-            _sample_workspaces[key] = workspace
+        workspace = _scratch(_sample_workspaces, need, hidden_states.device, sp, 1)      # born zeroed
     rc = lib.mux_greedy_sample(out.data_ptr(), hidden_states.data_ptr(), _rows(hidden_states, "hidden_states"),
                                hidden_states.shape[0], ri_ptr, num_rows, embedding.data_ptr(),
                                _rows(embedding, "embedding"), embedding.shape[0],
                                int(vocab_size), hidden_states.shape[1], _dtype_code(hidden_states),
-                               workspace.data_ptr(), workspace.numel(), _stream_ptr(stream))
+                               workspace.data_ptr(), workspace.numel(), sp)
     _lib.check_attn(rc, "mux_greedy_sample")
     return out[:num_rows]
 
@@ -358,7 +364,14 @@ class CUMaskedStream:
         self.torch_stream.synchronize()
 
     def close(self):
+        """Destroys the stream.  Scratch tensors this module allocated while the
+        stream was current are dropped first: they must not outlive the stream
+        they are tied to (nor be found again under a recycled handle value)."""
         if self.cuda_stream:
+            self.torch_stream.synchronize()
+            for cache in (_workspaces, _sample_workspaces):
+                for key in [k for k in cache if k[1] == self.cuda_stream]:
+                    del cache[key]
             _lib.attn().mux_stream_destroy(self.cuda_stream)
             self.cuda_stream = None
 
