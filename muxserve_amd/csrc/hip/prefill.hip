@@ -260,7 +260,9 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
       __syncthreads();
       if (t + 1 < n_tiles) load_tile();
     }
-    if (k0 > wq0 + 31) continue;         // every key of the tile is in this wave's future
+    // Nothing to compute: every key of the tile is in this wave's future, or all
+    // of the wave's rows are past the prompt's end.
+    if (k0 > wq0 + 31 || wq0 >= len) continue;
     const uint16_t *const Kt = DMA ? smem + cur * kTileElems : Ks;           // this tile's K
     const uint16_t *const Vr = DMA ? smem + (2 + cur) * kTileElems : Vt;     // this tile's V (row-major) or V^T
 
