@@ -7,7 +7,8 @@
 // registers:
 //     S^T[key][q] = K . Q^T      A = K tile   (LDS, row-major, 16-byte frags)
 //                                B = Q^T      (registers, loaded once)
-//     O^T[d][q]  += V^T . P^T    A = V^T tile (LDS, stored transposed)
+//     O^T[d][q]  += V^T . P^T    A = V^T      (the row-major V tile in LDS, read
+//                                              with the transposing LDS read)
 //                                B = P^T      = the S^T accumulators, converted
 // In the 32x32 accumulator layout a lane owns ONE query column (q = lane%32)
 // and 16 of the 32 keys of a block, so softmax statistics are per-lane scalars
@@ -16,8 +17,6 @@
 // B-operand fragments of the P.V products - provided the V^T fragments use the
 // same key order (two groups of four keys), which costs nothing because V^T is
 // read from LDS anyway.
-// V is transposed on its way into LDS: a thread loads 4 keys x 8 dims, does the
-// 4x8 16-bit transpose with byte permutes, and writes 8 rows of V^T.
 // The next tile's global loads are issued before the current tile's math.
 #include "mux_common.h"
 
@@ -31,8 +30,6 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kBM = 128;                 // query rows per workgroup
 constexpr int kBN = 64;                  // keys per tile
-constexpr int kKRow = kHeadSize + 8;     // K tile row length in elements (272 B: 16-byte frags, rows 4 banks apart)
-constexpr int kVRow = kBN + 4;           // V^T tile row length in elements (136 B: 8-byte frags, rows 2 banks apart)
 
 union Frag {
   u32x4 u;
@@ -77,14 +74,13 @@ struct PrefillParams {
   int32_t out_rows_16b;   // out and its row stride allow 16-byte stores
 };
 
-// DMA = true: K and V tiles go from global memory straight into LDS
+// K and V tiles go from global memory straight into LDS
 // (global_load_lds_dwordx4: lane l's 16 bytes land at base + 16 l), row-major
 // [key][128 dims] with the 16-byte chunks of a row XOR-swizzled by the row
 // number so that fragment reads spread over the banks; V^T fragments come out of
 // the row-major tile with the transposing read ds_read_b64_tr_b16.  No staging
-// registers, no LDS stores, no byte permutes; two tile buffers, one barrier per
-// tile.  DMA = false: the tiles are staged through registers, V transposed on
-// its way into LDS (kept for reference and comparison).
+// registers, no LDS stores, no byte permutes; two tile buffers per operand, one
+// barrier per tile.
 typedef short v4i16 __attribute__((ext_vector_type(4)));
 // A wave raises its issue priority while it feeds the matrix cores and drops
 // it for the softmax, so that of the two waves of a SIMD the one in its MFMA
@@ -94,15 +90,12 @@ typedef short v4i16 __attribute__((ext_vector_type(4)));
 #define MUX_PF_PRIO_VALU 0
 constexpr int kTileElems = kBN * kHeadSize;          // one unpadded row-major tile
 
-template <typename T, bool DMA>
+template <typename T>
 __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillParams P) {
   constexpr int D = kHeadSize;
-  // DMA: K[2], V[2] tile buffers.  Otherwise one buffer: the K tile, then the
-  // V^T tile.  The epilogue reuses the memory for the output rows.
-  constexpr int kSmemElems = DMA ? 4 * kTileElems : kBN * kKRow + D * kVRow;
+  // K[2], V[2] tile buffers.  The epilogue reuses the memory for the output rows.
+  constexpr int kSmemElems = 4 * kTileElems;
   __shared__ __attribute__((aligned(16))) uint16_t smem[kSmemElems];
-  uint16_t *const Ks = smem;
-  uint16_t *const Vt = smem + kBN * kKRow;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -162,65 +155,16 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
   // Rows past the prompt re-read its last row: finite data whose probability is
   // exactly 0 (such a key is in the future of every valid query).
 
-  // Register path.  K: thread takes chunk (key = tid/16 + 16 i, dchunk = tid%16).
-  // V: thread takes keys 4 kg .. 4 kg+3 (kg = tid%16) of dchunk vc = tid/16.
-  const int kc = tid & 15, kk = tid >> 4;
-  const int vg = tid & 15, vc = tid >> 4;
-  uint32_t koff[4], voff[DMA ? 1 : 4];
-  u32x4 kst[DMA ? 1 : 4], vst[DMA ? 1 : 4];
-  uint32_t kmax, vmax;
-  if constexpr (!DMA) {
+  // Instruction i of wave w fills KiB 4 i + w of a tile = rows 16 i + 4 w .. +3;
+  // lane l sits at row 16 i + 4 w + l/16, position l%16, and fetches chunk
+  // position ^ (row % 16) - the same chunk for every i.
+  uint32_t koff[4];
+  const int row0 = 4 * wave + (lane >> 4);
+  const int chunk0 = (lane & 15) ^ (row0 & 15);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      koff[i] = static_cast<uint32_t>(kk + 16 * i) * row_bytes + 16u * kc;
-      voff[i] = static_cast<uint32_t>(4 * vg + i) * row_bytes + 16u * vc;
-    }
-    kmax = last_row + 16u * kc;
-    vmax = last_row + 16u * vc;
-  } else {
-    // DMA path.  Instruction i of wave w fills KiB 4 i + w of a tile = rows
-    // 16 i + 4 w .. +3; lane l sits at row 16 i + 4 w + l/16, position l%16, and
-    // fetches chunk position ^ (row % 16) - the same chunk for every i.
-    const int row0 = 4 * wave + (lane >> 4);
-    const int chunk = (lane & 15) ^ (row0 & 15);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) koff[i] = static_cast<uint32_t>(row0 + 16 * i) * row_bytes + 16u * chunk;
-    kmax = last_row + 16u * chunk;
-    vmax = kmax;
-  }
-  auto load_tile = [&]() {                 // register path: loads the next tile in sequence
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      kst[i] = *reinterpret_cast<const u32x4 *>(kbase + min(koff[i], kmax));
-      koff[i] += tile_bytes;
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      vst[i] = *reinterpret_cast<const u32x4 *>(vbase + min(voff[i], vmax));
-      voff[i] += tile_bytes;
-    }
-  };
-  auto store_tile = [&]() {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      *reinterpret_cast<u32x4 *>(&Ks[(kk + 16 * i) * kKRow + 8 * kc]) = kst[i];
-    // 4 keys x 8 dims -> 8 rows of V^T, 4 keys (8 bytes) each.
-    const uint32_t a[4][4] = {{vst[0].x, vst[0].y, vst[0].z, vst[0].w},
-                              {vst[1].x, vst[1].y, vst[1].z, vst[1].w},
-                              {vst[2].x, vst[2].y, vst[2].z, vst[2].w},
-                              {vst[3].x, vst[3].y, vst[3].z, vst[3].w}};
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {        // dword w of a chunk holds dims 2w, 2w+1
-      // low halves -> dim 2w, high halves -> dim 2w+1
-      const uint32_t lo01 = __builtin_amdgcn_perm(a[1][w], a[0][w], 0x05040100u);
-      const uint32_t lo23 = __builtin_amdgcn_perm(a[3][w], a[2][w], 0x05040100u);
-      const uint32_t hi01 = __builtin_amdgcn_perm(a[1][w], a[0][w], 0x07060302u);
-      const uint32_t hi23 = __builtin_amdgcn_perm(a[3][w], a[2][w], 0x07060302u);
-      *reinterpret_cast<u32x2 *>(&Vt[(8 * vc + 2 * w) * kVRow + 4 * vg]) = u32x2{lo01, lo23};
-      *reinterpret_cast<u32x2 *>(&Vt[(8 * vc + 2 * w + 1) * kVRow + 4 * vg]) = u32x2{hi01, hi23};
-    }
-  };
-  auto dma_tile = [&](int buf) {           // DMA path: the next tile in sequence into buffer buf
+  for (int i = 0; i < 4; ++i) koff[i] = static_cast<uint32_t>(row0 + 16 * i) * row_bytes + 16u * chunk0;
+  const uint32_t kmax = last_row + 16u * chunk0;
+  auto dma_tile = [&](int buf) {           // the next tile in sequence into buffer buf
     typedef __attribute__((address_space(3))) void lds_void;
     typedef const __attribute__((address_space(1))) void global_void;
 #pragma unroll
@@ -243,28 +187,20 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
     v_lane_base[0] = rl * D + 8 * (cl ^ rl) + 4 * (m & 1);
     v_lane_base[1] = rl * D + 8 * (cl ^ rl ^ 4) + 4 * (m & 1);
   }
-  if constexpr (DMA) dma_tile(0);
-  else load_tile();
+  dma_tile(0);
   for (int t = 0; t < n_tiles; ++t) {
     const int k0 = t * kBN;
     const int cur = t & 1;
-    if constexpr (DMA) {
-      // This wave's part of tile t has landed; after the barrier all of it has,
-      // and everybody is done with the other buffer.
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
-      if (t + 1 < n_tiles) dma_tile(cur ^ 1);
-    } else {
-      __syncthreads();                     // everyone is done reading the previous tile
-      store_tile();
-      __syncthreads();
-      if (t + 1 < n_tiles) load_tile();
-    }
+    // This wave's part of tile t has landed; after the barrier all of it has,
+    // and everybody is done with the other buffer.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (t + 1 < n_tiles) dma_tile(cur ^ 1);
     // Nothing to compute: every key of the tile is in this wave's future, or all
     // of the wave's rows are past the prompt's end.
     if (k0 > wq0 + 31 || wq0 >= len) continue;
-    const uint16_t *const Kt = DMA ? smem + cur * kTileElems : Ks;           // this tile's K
-    const uint16_t *const Vr = DMA ? smem + (2 + cur) * kTileElems : Vt;     // this tile's V (row-major) or V^T
+    const uint16_t *const Kt = smem + cur * kTileElems;           // this tile's K
+    const uint16_t *const Vr = smem + (2 + cur) * kTileElems;     // this tile's V (row-major)
 
     // ---- S^T = K . Q^T : two 32-key blocks ------------------------------------------
     // LDS fragment reads run kDepth steps ahead of the MFMAs that consume them.
@@ -280,12 +216,8 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
       // Fragment j: key block j % 2, dims 16 (j / 2) + 8 half .. +7 of key row qcol.
       auto read_k = [&](int j) {
         Frag f;
-        if constexpr (DMA) {
-          const int row = 32 * (j % 2) + qcol, chunk = 2 * (j / 2) + half;
-          f.u = *reinterpret_cast<const u32x4 *>(Kt + row * D + 8 * (chunk ^ (row & 15)));
-        } else {
-          f.u = *reinterpret_cast<const u32x4 *>(Kt + (32 * (j % 2) + qcol) * kKRow + 16 * (j / 2) + 8 * half);
-        }
+        const int row = 32 * (j % 2) + qcol, chunk = 2 * (j / 2) + half;
+        f.u = *reinterpret_cast<const u32x4 *>(Kt + row * D + 8 * (chunk ^ (row & 15)));
         return f;
       };
       Frag ring[kDepth];
@@ -376,33 +308,26 @@ __global__ __launch_bounds__(256, 2) void prefill_causal_kernel(const PrefillPar
       auto read_v = [&](int n) {         // fragment n = 4 ks + mb
         const int mb = n % 4, ks = n / 4;
         Frag f;
-        if constexpr (DMA) {
-          // The transposing read works on groups of 16 lanes: lane 4 j + m of a
-          // group points at dims 4 m .. 4 m + 3 of key row j, and lane i of the
-          // group receives dim i of rows 0..3.  Here a group covers dims
-          // 32 mb + 16 (lane/16 % 2) .. +15 and keys 16 ks + 4 half (+ 8) .. +3.
-          // Address: row = 16 ks + 8 hsel + rl with rl = 4 half + jrow, chunk =
-          // 4 mb + cl, position = chunk ^ (row % 16) = (cl ^ rl) ^ 4 (mb ^ 2 hsel).
-          // The lane part cl ^ rl is below 8, so bit 3 of the constant part adds
-          // and only its bit 2 (mb odd) has to be folded into the lane's base:
-          // two bases per lane, everything else is an immediate offset.
-          typedef __attribute__((address_space(3))) v4i16 lds_v4i16;
-          u32x2 part[2];
+        // The transposing read works on groups of 16 lanes: lane 4 j + m of a
+        // group points at dims 4 m .. 4 m + 3 of key row j, and lane i of the
+        // group receives dim i of rows 0..3.  Here a group covers dims
+        // 32 mb + 16 (lane/16 % 2) .. +15 and keys 16 ks + 4 half (+ 8) .. +3.
+        // Address: row = 16 ks + 8 hsel + rl with rl = 4 half + jrow, chunk =
+        // 4 mb + cl, position = chunk ^ (row % 16) = (cl ^ rl) ^ 4 (mb ^ 2 hsel).
+        // The lane part cl ^ rl is below 8, so bit 3 of the constant part adds
+        // and only its bit 2 (mb odd) has to be folded into the lane's base:
+        // two bases per lane, everything else is an immediate offset.
+        typedef __attribute__((address_space(3))) v4i16 lds_v4i16;
+        u32x2 part[2];
 #pragma unroll
-          for (int hsel = 0; hsel < 2; ++hsel) {
-            const uint16_t *src = Vr + v_lane_base[mb & 1] + (16 * ks + 8 * hsel) * D + 64 * (((mb >> 1) ^ hsel) & 1);
-            const v4i16 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16 *)src);
-            union { v4i16 v; u32x2 u; } c;
-            c.v = r;
-            part[hsel] = c.u;
-          }
-          f.u = u32x4{part[0].x, part[0].y, part[1].x, part[1].y};
-        } else {
-          const uint16_t *r = Vr + (32 * mb + qcol) * kVRow + 4 * half + 16 * ks;
-          const u32x2 lo = *reinterpret_cast<const u32x2 *>(r);
-          const u32x2 hi = *reinterpret_cast<const u32x2 *>(r + 8);
-          f.u = u32x4{lo.x, lo.y, hi.x, hi.y};
+        for (int hsel = 0; hsel < 2; ++hsel) {
+          const uint16_t *src = Vr + v_lane_base[mb & 1] + (16 * ks + 8 * hsel) * D + 64 * (((mb >> 1) ^ hsel) & 1);
+          const v4i16 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16 *)src);
+          union { v4i16 v; u32x2 u; } c;
+          c.v = r;
+          part[hsel] = c.u;
         }
+        f.u = u32x4{part[0].x, part[0].y, part[1].x, part[1].y};
         return f;
       };
       Frag ring[kDepth];
@@ -510,9 +435,8 @@ extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const v
   if (n_wg > 0x7fffffff) return MUXA_EUNSUPPORTED;
   const dim3 grid(static_cast<uint32_t>(n_wg));
   hipStream_t st = static_cast<hipStream_t>(stream);
-  constexpr bool kDma = true;
-  if (dtype == MUXA_DTYPE_F16) hipLaunchKernelGGL((prefill_causal_kernel<F16, kDma>), grid, dim3(256), 0, st, P);
-  else hipLaunchKernelGGL((prefill_causal_kernel<BF16, kDma>), grid, dim3(256), 0, st, P);
+  if (dtype == MUXA_DTYPE_F16) hipLaunchKernelGGL((prefill_causal_kernel<F16>), grid, dim3(256), 0, st, P);
+  else hipLaunchKernelGGL((prefill_causal_kernel<BF16>), grid, dim3(256), 0, st, P);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e);
   return MUXA_OK;
