@@ -35,7 +35,7 @@ struct StepParams {
 __device__ __forceinline__ bool desc_ok(const StepParams &P, const int32_t *d) {
   const int64_t count = static_cast<int64_t>(d[3]) * P.per;
   return d[0] >= 0 && d[0] < P.max_rows && d[1] >= 0 && d[1] <= P.max_blocks_per_seq && d[2] >= 0 && d[3] >= 0 &&
-         d[2] + d[3] <= d[1] && d[4] >= 1 && d[4] + count <= P.n_block_info && d[5] >= 0 && d[6] >= 0;
+         static_cast<int64_t>(d[2]) + d[3] <= d[1] && d[4] >= 1 && d[4] + count <= P.n_block_info && d[5] >= 0 && d[6] >= 0;
 }
 
 __global__ __launch_bounds__(256) void step_append_kernel(const StepParams P) {
@@ -126,7 +126,9 @@ extern "C" int32_t mux_build_step_inputs(int32_t *mirror, int32_t max_rows, int3
   if (!desc || !block_info || (num_tokens > 0 && !slot_mapping) || (max_blocks_out > 0 && !block_tables))
     return MUXA_EINVAL;
   const int64_t per = static_cast<int64_t>(num_layers) * num_heads;
-  if (per > 0x7fffffff / 4 || num_seqs > 65535 || static_cast<int64_t>(max_new_blocks) * per > (int64_t{1} << 40))
+  // Grid limits: y and z dimensions hold at most 65535 workgroups.
+  if (per > 65535 * 1024 || num_seqs > 65535 || max_blocks_out > 65535 * 64 ||
+      static_cast<int64_t>(max_new_blocks) * per > (int64_t{1} << 40))
     return MUXA_EUNSUPPORTED;
   StepParams P;
   P.mirror = mirror;

@@ -91,3 +91,46 @@ def test_device_built_step_inputs_with_preemption():
         alive = [r for r in alive if r not in cut]
         if not alive:
             break
+
+
+def test_descriptors_that_do_not_fit_are_skipped():
+    """Descriptors pointing outside the mirror or the reply (row, block count,
+    first new block, reply offset, sums that wrap in 32 bits) leave the mirror,
+    the slots of their tokens and their table rows alone; the one well-formed
+    descriptor among them is still carried out."""
+    print("[case] device step inputs, malformed descriptors", flush=True)
+    from muxserve_amd import _lib
+    L, H, bs, rows, max_blk = 2, 3, 16, 4, 8
+    per = L * H
+    big = 2 ** 31 - 1
+    mirror = torch.full((rows, max_blk, L, H), -7, dtype=torch.int32, device=DEV)
+    reply = torch.arange(100, 100 + 1 + 2 * per, dtype=torch.int32)       # [preempt idx | 2 blocks of ids]
+    # row, blocks, first new, new, reply offset, length, first token, decoding
+    desc = torch.tensor([
+        [rows, 1, 0, 1, 1, 5, 0, 0],            # row outside the mirror
+        [0, max_blk + 1, 0, 1, 1, 5, 5, 0],     # more blocks than a row holds
+        [0, 2, big, 1, 1, 5, 10, 0],            # first new + new wraps around
+        [0, 2, 0, 2, 1 + per, 5, 15, 0],        # reply too short for the new blocks
+        [0, 2, 1, 2, 1, 5, 20, 0],              # new blocks reach past the run
+        [1, 2, 0, 2, 1, 20, 25, 0],             # well-formed: 20 prompt tokens, 2 new blocks
+        [0, 1, 0, 0, 1, -3, 45, 1],             # negative length
+    ], dtype=torch.int32)
+    num_tokens = 50
+    slots = torch.full((num_tokens, L, H), -1, dtype=torch.int64, device=DEV)
+    tables = torch.full((L, desc.shape[0], H, max_blk), -9, dtype=torch.int32, device=DEV)
+    d_desc, d_reply = desc.to(DEV), reply.to(DEV)
+    rc = _lib.attn().mux_build_step_inputs(
+        mirror.data_ptr(), rows, max_blk, L, H, bs, d_desc.data_ptr(), desc.shape[0], d_reply.data_ptr(),
+        reply.numel(), 2, num_tokens, slots.data_ptr(), tables.data_ptr(), max_blk,
+        torch.cuda.current_stream().cuda_stream)
+    _lib.check_attn(rc, "mux_build_step_inputs")
+    torch.cuda.synchronize()
+    want_mirror = torch.full((rows, max_blk, L, H), -7, dtype=torch.int32)
+    want_mirror[1, :2] = reply[1:].view(2, L, H)
+    assert torch.equal(mirror.cpu(), want_mirror)
+    want_slots = torch.full((num_tokens, L, H), -1, dtype=torch.int64)
+    for k in range(20):
+        want_slots[25 + k] = want_mirror[1, k // bs].long() * bs + k % bs
+    assert torch.equal(slots.cpu(), want_slots)
+    # no descriptor here is a decode step: every table row is defined and empty
+    assert (tables.cpu() == 0).all()
