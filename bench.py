@@ -594,7 +594,7 @@ def main():
         calls = [ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
                                 total_context_len=0 if args.no_hint else int(m.context_lens.sum()))
                  for m in models]
-        sets.append((models, calls))
+        sets.append((models, calls, torch.from_numpy(used.astype(np.int32)).to(dev)))
     torch.cuda.synchronize()
 
     def step(i):
@@ -619,9 +619,17 @@ def main():
     ev_ms = ev0.elapsed_time(ev1) / args.steps
     ms = max(wall_ms, ev_ms)
 
+    # The yardstick: the same blocks read by the bare gather-read probe (the decode
+    # kernel's loads, no table walk, no arithmetic), same rotation of the sets.
+    sink = torch.zeros((1,), dtype=torch.int32, device=dev)
+    probe_ms = _time(lambda i: ops.probe_gather_read(k_pool, v_pool, sets[i % len(sets)][2], sink),
+                     args.steps, args.warmup)
+    probe_bytes = sum(int(s[2].numel()) * 8192 * v for s, v in
+                      zip(sets, [len(range(i, args.steps, len(sets))) for i in range(len(sets))])) / args.steps
+
     tokens = sum(m.batch for m in sets[0][0])
     step_bytes = [sum(workloads.decode_bytes(m.context_lens, m.num_q_heads, m.num_kv_heads, bs) for m in models)
-                  for models, _ in sets]
+                  for models, _, _ in sets]
     visits = [len(range(i, args.steps, len(sets))) for i in range(len(sets))]
     avg_bytes = sum(b * v for b, v in zip(step_bytes, visits)) / max(1, sum(visits))
     achieved = avg_bytes / (ev_ms * 1e-3) / 1e9
@@ -656,6 +664,9 @@ def main():
             "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiles/paged_decode_mixed3_hbm_traffic.txt",
             "kernel": "paged_decode_kernel<F16,16,1,4>",
             "event_ms_per_step": ev_ms,
+            "bare_gather_read_of_the_same_blocks": {
+                "ms": probe_ms, "bytes": int(probe_bytes), "GB/s": probe_bytes / (probe_ms * 1e-3) / 1e9,
+                "kernel": "probe_gather_read_kernel (whole 4 KiB blocks, no arithmetic)"},
         },
     }
     if not args.no_cpu_baseline:

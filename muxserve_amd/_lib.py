@@ -140,6 +140,7 @@ ATTN_SIGNATURES = {
                                   c_vp, c_sz, c_vp]),
     "mux_build_step_inputs": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_i32, c_vp, c_i64, c_i32,
                                       c_i32, c_vp, c_vp, c_i32, c_vp]),
+    "mux_probe_gather_read": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp]),
     "mux_stream_create_cu_range": (c_i32, [c_vp, c_i32, c_i32, c_vp]),
     "mux_stream_destroy": (c_i32, [c_vp]),
     "mux_device_cu_info": (c_i32, [c_vp]),

@@ -22,7 +22,7 @@ ATTN_LIB = os.path.join(PKG, "libmuxattn.so")
 HOST_SOURCES = [os.path.join(CSRC, "host", f) for f in ("kv_storage.cpp", "batch_scheduler.cpp")]
 HIP_SOURCES = [os.path.join(CSRC, "hip", f) for f in (
     "cache_write.hip", "paged_decode.hip", "prefill.hip", "rotary.hip", "model_ops.hip", "sampler.hip",
-    "step_tables.hip", "runtime.hip")]
+    "step_tables.hip", "probe.hip", "runtime.hip")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # Packed-FP32 instruction selection is switched off for every device

@@ -473,3 +473,28 @@ def test_decode_is_invariant_under_relabelling_of_the_physical_blocks(Hq, Hkv, d
         torch.cuda.synchronize()
         outs.append(out[:B].cpu().view(torch.int16))
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
+def test_gather_read_probe_runs_and_rejects_what_it_cannot_read():
+    """The measuring aid next to the decode kernel: accepts any id list
+    (duplicates, ids outside the pool are clamped, lengths that are no multiple
+    of a wave's four blocks), never writes the pools, refuses other block sizes."""
+    print("[case] gather-read probe", flush=True)
+    from muxserve_amd import _lib
+    N = 512
+    k_pool, v_pool = allocate_gpu_cache(N, 16, DEV)
+    k_pool.normal_()
+    v_pool.normal_()
+    k0, v0 = k_pool.clone(), v_pool.clone()
+    sink = torch.zeros((1,), dtype=torch.int32, device=DEV)
+    for n in (1, 3, 4, 17, 1000):
+        ids = torch.randint(-5, N + 5, (n,), dtype=torch.int32, device=DEV)
+        ops.probe_gather_read(k_pool, v_pool, ids, sink)
+    ops.probe_gather_read(k_pool, v_pool, torch.zeros((0,), dtype=torch.int32, device=DEV), sink)
+    torch.cuda.synchronize()
+    assert torch.equal(k_pool, k0) and torch.equal(v_pool, v0)
+    k8, v8 = allocate_gpu_cache(64, 8, DEV)
+    with pytest.raises(RuntimeError):
+        ops.probe_gather_read(k8, v8, torch.zeros((4,), dtype=torch.int32, device=DEV), sink)
+    assert _lib.attn().mux_probe_gather_read(None, v_pool.data_ptr(), N, sink.data_ptr(), 4, 16, sink.data_ptr(),
+                                             None) == -1      # MUXA_EINVAL
