@@ -53,7 +53,7 @@ def test_scenario_definitions_match_fixture():
     assert _GOLD["random_05"]["scenario"] == scenarios.random_scenario(5)
 
 
-@pytest.mark.parametrize("seed", range(100, 140))
+@pytest.mark.parametrize("seed", range(100, 300))
 def test_product_matches_oracle_on_fresh_random_scenarios(seed):
     sc = scenarios.random_scenario(seed)
     a = scenarios.run_scenario(host_oracle.KVStorage, host_oracle.BatchScheduler, sc)
@@ -65,12 +65,22 @@ _REF = build_ref.load() if os.path.isdir(os.path.join(os.path.dirname(build_ref.
 
 
 @pytest.mark.skipif(_REF[0] is None, reason="oracle/_ref not built (needs the reference checkout)")
-@pytest.mark.parametrize("seed", range(200, 230))
+@pytest.mark.parametrize("seed", range(200, 320))
 def test_oracle_matches_live_compiled_reference(seed):
     sc = scenarios.random_scenario(seed)
     mm, bsm = _REF
     a = scenarios.run_scenario(mm.KVStorage, bsm.BatchScheduler, sc)
     b = scenarios.run_scenario(host_oracle.KVStorage, host_oracle.BatchScheduler, sc)
+    assert a == b, _first_diff(a, b)
+
+
+@pytest.mark.skipif(_REF[0] is None, reason="oracle/_ref not built (needs the reference checkout)")
+@pytest.mark.parametrize("seed", range(400, 460))
+def test_product_matches_live_compiled_reference(seed):
+    sc = scenarios.random_scenario(seed)
+    mm, bsm = _REF
+    a = scenarios.run_scenario(mm.KVStorage, bsm.BatchScheduler, sc)
+    b = scenarios.run_scenario(KVStorage, BatchScheduler, sc)
     assert a == b, _first_diff(a, b)
 
 
