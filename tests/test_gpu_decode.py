@@ -498,3 +498,29 @@ def test_gather_read_probe_runs_and_rejects_what_it_cannot_read():
         ops.probe_gather_read(k8, v8, torch.zeros((4,), dtype=torch.int32, device=DEV), sink)
     assert _lib.attn().mux_probe_gather_read(None, v_pool.data_ptr(), N, sink.data_ptr(), 4, 16, sink.data_ptr(),
                                              None) == -1      # MUXA_EINVAL
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_decode_random_shapes_against_the_oracle(seed):
+    """Seeded draws over head grouping, block size, storage type, partition size,
+    layer slice and context lengths (short, around tile and partition boundaries,
+    long), each against the oracle at the 2e-3 bar."""
+    rng = np.random.Generator(np.random.PCG64(1000 + seed))
+    Hkv = int(rng.choice([1, 2, 3, 5]))
+    ratio = int(rng.choice([1, 1, 2, 4, 8, 16, 3]))
+    bs = int(rng.choice([8, 16, 16, 32]))
+    dtype = [torch.float16, torch.bfloat16][int(rng.integers(2))]
+    partition = int(rng.choice([0, 64, 128, 256, 512]))
+    B = int(rng.integers(1, 12))
+    kinds = rng.integers(0, 4, size=B)
+    ctx = np.where(kinds == 0, rng.integers(1, 20, size=B),
+                   np.where(kinds == 1, 64 * rng.integers(1, 9, size=B) + rng.integers(-1, 2, size=B),
+                            np.where(kinds == 2, rng.integers(1, 600, size=B), rng.integers(600, 1500, size=B))))
+    L = int(rng.integers(1, 4))
+    layer = int(rng.integers(L))
+    _announce(f"decode random seed={seed} Hq={Hkv * ratio} Hkv={Hkv} bs={bs} {dtype} partition={partition} "
+              f"L={L} layer={layer} ctx={ctx.tolist()}")
+    got, want = _decode_case(2000 + seed, ctx.tolist(), Hkv * ratio, Hkv, bs, dtype=dtype, partition=partition,
+                             num_layers=L, layer=layer, q_in_qkv=bool(rng.integers(2)), hint=bool(rng.integers(2)),
+                             repeat=2)
+    _check(got, want, out_dtype=dtype)
