@@ -27,7 +27,9 @@
  * (a hipStream_t passed as void*; NULL = the default stream) and the call
  * returns without synchronising.  Return value: 0 on success, a negative
  * MUXA_E* code on a rejected argument; no exceptions cross the boundary.
- * Shapes are validated on the host before any launch.
+ * Shapes are validated on the host before any launch.  A call with nothing to
+ * do (no tokens, sequences, prompts or rows) returns MUXA_OK without a launch,
+ * and the data pointers of such a call may be NULL.
  */
 #ifndef MUXSERVE_ATTN_H
 #define MUXSERVE_ATTN_H

@@ -287,7 +287,8 @@ int32_t check_cache_write(const void *k, const void *v, int64_t kv_row_stride, c
                           const void *v_pool, int64_t num_pool_blocks, const int64_t *slot_mapping, int32_t layer,
                           int32_t num_layers, int32_t num_tokens, int32_t num_kv_heads, int32_t head_size,
                           int32_t block_size, int32_t dtype) {
-  if (!k || !v || !k_pool || !v_pool || !slot_mapping) return MUXA_EINVAL;
+  // (pointers are only required when there is something to do)
+  if (num_tokens > 0 && (!k || !v || !k_pool || !v_pool || !slot_mapping)) return MUXA_EINVAL;
   if (num_tokens < 0 || num_kv_heads <= 0 || num_pool_blocks <= 0) return MUXA_EINVAL;
   if (layer < 0 || layer >= num_layers) return MUXA_EINVAL;
   if (head_size != kHeadSize) return MUXA_EUNSUPPORTED;
@@ -340,7 +341,7 @@ extern "C" int32_t mux_rope_reshape_and_cache(const int64_t *positions, void *q,
   const int32_t rc = check_cache_write(k, v, kv_row_stride, k_pool, v_pool, num_pool_blocks, slot_mapping, layer,
                                        num_layers, num_tokens, num_kv_heads, head_size, block_size, dtype);
   if (rc != MUXA_OK) return rc;
-  if (!positions || !cos_sin || max_position <= 0) return MUXA_EINVAL;
+  if ((num_tokens > 0 && (!positions || !cos_sin)) || max_position <= 0) return MUXA_EINVAL;
   if (rotary_dim != kHeadSize) return MUXA_EUNSUPPORTED;   // partial rotation: use mux_rotary_neox + mux_reshape_and_cache
   if (q != nullptr) {
     if (num_q_heads <= 0 || num_q_heads % num_kv_heads != 0) return MUXA_EINVAL;

@@ -167,7 +167,8 @@ extern "C" int32_t mux_rms_norm(void *out, int64_t out_row_stride, const void *x
                                 const void *weight, float eps, int32_t num_tokens, int32_t hidden_size,
                                 int32_t dtype, void *stream) {
   using namespace mux;
-  if (!out || !x || !weight) return MUXA_EINVAL;
+  // (pointers are only required when there is something to do)
+  if (num_tokens > 0 && (!out || !x || !weight)) return MUXA_EINVAL;
   if (num_tokens < 0 || hidden_size <= 0 || !(eps >= 0.f)) return MUXA_EINVAL;
   if (dtype != MUXA_DTYPE_F16 && dtype != MUXA_DTYPE_BF16) return MUXA_EUNSUPPORTED;
   if (hidden_size % 8) return MUXA_EUNSUPPORTED;
@@ -211,7 +212,7 @@ extern "C" int32_t mux_rms_norm(void *out, int64_t out_row_stride, const void *x
 extern "C" int32_t mux_silu_and_mul(void *out, int64_t out_row_stride, const void *x, int64_t x_row_stride,
                                     int32_t num_tokens, int32_t d, int32_t dtype, void *stream) {
   using namespace mux;
-  if (!out || !x) return MUXA_EINVAL;
+  if (num_tokens > 0 && (!out || !x)) return MUXA_EINVAL;
   if (num_tokens < 0 || d <= 0) return MUXA_EINVAL;
   if (dtype != MUXA_DTYPE_F16 && dtype != MUXA_DTYPE_BF16) return MUXA_EUNSUPPORTED;
   if (d % 8) return MUXA_EUNSUPPORTED;

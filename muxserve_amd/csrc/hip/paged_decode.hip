@@ -1095,7 +1095,8 @@ hipError_t launch_bs(int BS, int G, const DecodeParams &P, int grid, hipStream_t
 }
 
 int32_t validate_item(const MuxDecodeItem &it, int block_size) {
-  if (!it.out || !it.q || !it.block_tables || !it.context_lens) return MUXA_EINVAL;
+  // (pointers are only required when the item has sequences)
+  if (it.num_seqs > 0 && (!it.out || !it.q || !it.block_tables || !it.context_lens)) return MUXA_EINVAL;
   if (it.num_seqs < 0 || it.num_q_heads <= 0 || it.num_kv_heads <= 0) return MUXA_EINVAL;
   if (it.num_q_heads % it.num_kv_heads != 0) return MUXA_EINVAL;
   if (it.layer < 0 || it.layer >= it.num_layers) return MUXA_EINVAL;

@@ -398,7 +398,9 @@ extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const v
                                       int32_t max_prompt_len, int32_t num_q_heads, int32_t num_kv_heads,
                                       int32_t head_size, float scale, int32_t dtype, void *stream) {
   using namespace mux;
-  if (!out || !q || !k || !v || !cu_seqlens) return MUXA_EINVAL;
+  // (pointers are only required when there is something to do)
+  const bool work = num_prompts > 0 && max_prompt_len > 0;
+  if (work && (!out || !q || !k || !v || !cu_seqlens)) return MUXA_EINVAL;
   if (num_prompts < 0 || max_prompt_len < 0 || num_q_heads <= 0 || num_kv_heads <= 0) return MUXA_EINVAL;
   if (num_q_heads % num_kv_heads != 0) return MUXA_EINVAL;
   if (head_size != kHeadSize) return MUXA_EUNSUPPORTED;

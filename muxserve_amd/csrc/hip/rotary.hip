@@ -59,7 +59,8 @@ extern "C" int32_t mux_rotary_neox(const int64_t *positions, void *q, int64_t q_
                                    int32_t rotary_dim, int32_t num_tokens, int32_t num_q_heads,
                                    int32_t num_kv_heads, int32_t head_size, int32_t dtype, void *stream) {
   using namespace mux;
-  if (!positions || !q || !k || !cos_sin) return MUXA_EINVAL;
+  // (pointers are only required when there is something to do)
+  if (num_tokens > 0 && (!positions || !q || !k || !cos_sin)) return MUXA_EINVAL;
   if (num_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_position <= 0) return MUXA_EINVAL;
   if (head_size != kHeadSize) return MUXA_EUNSUPPORTED;
   if (rotary_dim <= 0 || rotary_dim > kHeadSize || rotary_dim % 4 != 0) return MUXA_EUNSUPPORTED;

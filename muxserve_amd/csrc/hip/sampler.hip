@@ -341,7 +341,8 @@ extern "C" int32_t mux_greedy_sample(int64_t *next_tokens, const void *hidden_st
                                      int32_t hidden_size, int32_t dtype, void *workspace, size_t workspace_bytes,
                                      void *stream) {
   using namespace mux;
-  if (!next_tokens || !hidden_states || !embedding) return MUXA_EINVAL;
+  // (pointers are only required when there is something to do)
+  if (num_rows > 0 && (!next_tokens || !hidden_states || !embedding)) return MUXA_EINVAL;
   if (num_rows < 0 || vocab_size <= 0 || hidden_size <= 0 || embedding_rows < vocab_size) return MUXA_EINVAL;
   if (num_hidden_rows < 1 || (!row_index && num_rows > num_hidden_rows)) return MUXA_EINVAL;
   if (dtype != MUXA_DTYPE_F16 && dtype != MUXA_DTYPE_BF16) return MUXA_EUNSUPPORTED;

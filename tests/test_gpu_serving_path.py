@@ -156,3 +156,34 @@ def test_fused_rotary_cache_write_equals_the_two_kernels(dtype, Hq, Hkv, bs):
     for a, b, what in zip(results[0], results[1], ("qkv rows", "k pool", "v pool")):
         assert torch.equal(a, b), f"{what} differ between the fused launch and the two kernels"
     assert torch.equal(results[1][0][T:], qkv.cpu().view(torch.int16)[T:]), "padding rows must not be touched"
+
+
+def test_empty_steps_are_accepted():
+    """No tokens, no sequences, no prompts, no sampled rows: every entry point
+    returns without launching and without touching its outputs."""
+    print("[case] empty steps", flush=True)
+    from muxserve_amd.attention import build_cos_sin_cache
+    H, bs, N = 2, 16, 64
+    k_pool, v_pool = allocate_gpu_cache(N, bs, DEV)
+    k_pool.fill_(3.0)
+    v_pool.fill_(3.0)
+    e16 = torch.empty((0, H * D), dtype=torch.float16, device=DEV)
+    slots = torch.empty((0, 1, H), dtype=torch.int64, device=DEV)
+    pos = torch.empty((0,), dtype=torch.int64, device=DEV)
+    cos_sin = build_cos_sin_cache(D, 64, 10000.0, DEV)
+    ops.reshape_and_cache(e16, e16, k_pool, v_pool, slots)
+    ops.rotary_neox(pos, e16, e16, cos_sin)
+    ops.rope_reshape_and_cache(pos, e16, e16, e16, cos_sin, k_pool, v_pool, slots)
+    # a padded batch whose valid part is empty
+    pad = torch.full((8, H * D), 5.0, dtype=torch.float16, device=DEV)
+    ops.reshape_and_cache(pad, pad, k_pool, v_pool, torch.zeros((8, 1, H), dtype=torch.int64, device=DEV), num_tokens=0)
+    out = torch.full((8, H * D), 7.0, dtype=torch.float16, device=DEV)
+    ops.paged_decode(out, pad, k_pool, v_pool, torch.empty((1, 0, H, 4), dtype=torch.int32, device=DEV),
+                     torch.empty((0,), dtype=torch.int32, device=DEV), 0, D ** -0.5)
+    ops.prefill_causal(out, pad, pad, pad, torch.zeros((1,), dtype=torch.int32, device=DEV), 0, D ** -0.5, H)
+    assert ops.rms_norm(e16[:, :64], torch.ones((64,), dtype=torch.float16, device=DEV), 1e-6).shape == (0, 64)
+    assert ops.silu_and_mul(e16).shape == (0, H * D // 2)
+    emb = torch.zeros((32, 256), dtype=torch.float16, device=DEV)
+    assert ops.greedy_sample(emb, torch.zeros((8, 256), dtype=torch.float16, device=DEV), 32, 0).shape == (0,)
+    torch.cuda.synchronize()
+    assert (out == 7.0).all() and (k_pool == 3.0).all() and (v_pool == 3.0).all()
