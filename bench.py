@@ -54,6 +54,8 @@ def parse():
     ap.add_argument("--no-hint", action="store_true", help="do not pass the host-side sum of context lengths")
     ap.add_argument("--no-prompt-order", action="store_true",
                     help="prefill3: start the prompts' workgroups as packed instead of longest first")
+    ap.add_argument("--no-prompt-lens", action="store_true",
+                    help="prefill3: do not pass the host-side prompt lengths (grid sized by the longest prompt)")
     ap.add_argument("--unfused", action="store_true", help="one launch per model instead of one fused launch")
     ap.add_argument("--workload", default="mixed3_decode",
                     choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long", "model_ops", "host_step"],
@@ -156,10 +158,14 @@ def bench_prefill3(args):
         wbytes += workloads.cache_write_bytes(T, Hkv)
         tokens += T
 
+    import ctypes
+    lens_of = {w[0].name: (ctypes.c_int32 * len(w[0].prompt_lens))(*[int(x) for x in w[0].prompt_lens]) for w in work}
+
     def attn(_):
         for m, q, k, v, out, cu, slots, T, order in work:
             ops.prefill_causal(out, q, k, v, cu, int(m.prompt_lens.max()), m.scale, m.num_kv_heads,
-                               prompt_order=None if args.no_prompt_order else order)
+                               prompt_order=None if args.no_prompt_order else order,
+                               prompt_lens=None if (args.no_prompt_lens or args.no_prompt_order) else lens_of[m.name])
 
     def write(_):
         for m, q, k, v, out, cu, slots, T, order in work:

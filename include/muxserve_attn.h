@@ -158,11 +158,18 @@ int32_t mux_paged_decode(void *out, int64_t out_row_stride, const void *q, int64
  * int32 [num_prompts], a permutation of the prompts - the order in which their
  * workgroups are started (the caller knows the lengths on the host; longest
  * first keeps the longest prompt off the end of the launch); NULL: as packed.
- * Results do not depend on it. */
+ * prompt_lens_host: optional HOST int32 [num_prompts], the prompt lengths the
+ * caller holds on the host anyway (InputMetadata.prompt_lens,
+ * pipeworker.py:81-90; each <= max_prompt_len).  With them the launch holds
+ * only the query tiles that exist, the heaviest of the whole batch first, and
+ * prompt_order is not used; batches of more than 896 query tiles of 128 rows
+ * fall back to the grid sized by max_prompt_len.  The device-side cu_seqlens
+ * stay authoritative for addresses and lengths.  Results depend on neither. */
 int32_t mux_prefill_causal(void *out, int64_t out_row_stride,
                            const void *q, int64_t q_row_stride,
                            const void *k, const void *v, int64_t kv_row_stride,
-                           const int32_t *cu_seqlens, const int32_t *prompt_order, int32_t num_prompts,
+                           const int32_t *cu_seqlens, const int32_t *prompt_order,
+                           const int32_t *prompt_lens_host, int32_t num_prompts,
                            int32_t max_prompt_len, int32_t num_q_heads, int32_t num_kv_heads,
                            int32_t head_size, float scale, int32_t dtype, void *stream);
 

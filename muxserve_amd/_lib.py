@@ -126,7 +126,7 @@ ATTN_SIGNATURES = {
     "mux_paged_decode": (c_i32, [c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_vp,
                                  c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32,
                                  c_f32, c_i32, c_i32, c_vp, c_sz, c_vp]),
-    "mux_prefill_causal": (c_i32, [c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_vp, c_i32, c_i32,
+    "mux_prefill_causal": (c_i32, [c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_i32, c_i32,
                                    c_i32, c_i32, c_i32, c_f32, c_i32, c_vp]),
     "mux_rotary_neox": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32,
                                 c_i32, c_vp]),

@@ -47,6 +47,7 @@ class InputMetadata:
     _cu_seqlens: Optional[torch.Tensor] = field(default=None, repr=False)
     _prompt_order: Optional[torch.Tensor] = field(default=None, repr=False)
     _last_rows: Optional[torch.Tensor] = field(default=None, repr=False)
+    _lens_array: Any = field(default=None, repr=False)
 
     def __post_init__(self):
         self.prompt_lens = [int(x) for x in self.prompt_lens]
@@ -78,6 +79,14 @@ class InputMetadata:
                 rows.append(end - 1)
             self._last_rows = torch.tensor(rows, dtype=torch.int32, device=device)
         return self._last_rows
+
+    def prompt_lens_array(self):
+        """The prompt lengths as a host int32 array for the C ABI, built once per
+        step and shared by every layer."""
+        if self._lens_array is None:
+            import ctypes
+            self._lens_array = (ctypes.c_int32 * len(self.prompt_lens))(*self.prompt_lens)
+        return self._lens_array
 
     def prompt_order(self, device) -> torch.Tensor:
         """int32 [num_prompts] on the device: the prompts longest first (the order
@@ -146,7 +155,7 @@ class PagedAttention(torch.nn.Module):
         if n_prompt > 0:
             ops.prefill_causal(out[:n_prompt], query[:n_prompt], key[:n_prompt], value[:n_prompt],
                                md.cu_seqlens(query.device), md.max_prompt_len, self.scale, self.num_kv_heads,
-                               prompt_order=md.prompt_order(query.device))
+                               prompt_lens=md.prompt_lens_array())
         if md.num_generation_tokens > 0:
             if key_cache is None or value_cache is None:
                 raise ValueError("decode needs the KV pool")

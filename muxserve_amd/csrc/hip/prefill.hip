@@ -35,6 +35,9 @@ constexpr int kBM = 128;                 // query rows per workgroup
 constexpr int kBN = 32;                  // keys per tile
 constexpr int kNKB = kBN / 32;           // 32-key blocks (one MFMA row block) per tile
 
+// Query tiles listed in the kernel argument (its size limit is 4 KiB).
+constexpr int kMaxPairs = 896;
+
 union Frag {
   u32x4 u;
   v8f16 h;
@@ -76,6 +79,11 @@ struct PrefillParams {
   int32_t num_groups;     // (prompt, kv head) pairs
   float scale_log2;
   int32_t out_rows_16b;   // out and its row stride allow 16-byte stores
+  // Compact grid (the caller gave the prompt lengths on the host): the query
+  // tiles that exist, heaviest first, as prompt << 16 | tile; 0 pairs = dense grid.
+  int32_t n_pairs;
+  int32_t kv_per_xcd;     // ceil(num_kv_heads / 8)
+  uint32_t pairs[kMaxPairs];
 };
 
 // K and V tiles go from global memory straight into LDS
@@ -107,23 +115,42 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // Workgroups are dealt to the 8 XCDs round-robin by id, and each XCD has its
   // own L2.  All workgroups that read the same K/V - the query tiles and query
-  // heads of one (prompt, kv head) group - are therefore given ids that are
-  // equal mod 8, and groups go round-robin over the XCDs.
-  const int per_group = P.ratio * P.q_tiles;
+  // heads of one (prompt, kv head) pair - are therefore given ids that are equal
+  // mod 8.
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int group = (slot / per_group) * 8 + xcd;
-  if (group >= P.num_groups) return;
-  const int in_group = slot % per_group;
-  const int prompt_rank = group / P.num_kv_heads;
-  // (an entry outside the batch is clamped: a malformed order costs results, never a stray read)
-  const int prompt =
-      P.prompt_order ? min(max(P.prompt_order[prompt_rank], 0), P.num_groups / P.num_kv_heads - 1) : prompt_rank;
-  const int hk = group % P.num_kv_heads;
-  const int hq = hk * P.ratio + in_group / P.q_tiles;
+  const int num_prompts = P.num_groups / P.num_kv_heads;
+  int prompt, hk, hq, q0;
+  if (P.n_pairs > 0) {
+    // Compact grid: only query tiles that exist, the heaviest of the whole batch
+    // first; kv head hk of prompt p lives on XCD (hk + p) % 8 (rotated by the
+    // prompt so that head counts that are no multiple of 8 load the XCDs evenly).
+    const int per_pair = P.kv_per_xcd * P.ratio;
+    const int pi = slot / per_pair;
+    if (pi >= P.n_pairs) return;
+    const int rem = slot - pi * per_pair;
+    const uint32_t pair = P.pairs[pi];
+    // (clamped: a malformed list costs results, never a stray read)
+    prompt = min(static_cast<int>(pair >> 16), num_prompts - 1);
+    q0 = static_cast<int>(pair & 0xffffu) * kBM;
+    hk = ((xcd - prompt) & 7) + 8 * (rem / P.ratio);
+    if (hk >= P.num_kv_heads) return;
+    hq = hk * P.ratio + rem % P.ratio;
+  } else {
+    // Dense grid: every prompt gets the tiles of the longest one, heaviest first;
+    // (prompt, kv head) groups go round-robin over the XCDs.
+    const int per_group = P.ratio * P.q_tiles;
+    const int group = (slot / per_group) * 8 + xcd;
+    if (group >= P.num_groups) return;
+    const int in_group = slot % per_group;
+    const int prompt_rank = group / P.num_kv_heads;
+    // (an entry outside the batch is clamped, as above)
+    prompt = P.prompt_order ? min(max(P.prompt_order[prompt_rank], 0), num_prompts - 1) : prompt_rank;
+    hk = group % P.num_kv_heads;
+    hq = hk * P.ratio + in_group / P.q_tiles;
+    q0 = (P.q_tiles - 1 - in_group % P.q_tiles) * kBM;
+  }
   const int seq_begin = P.cu_seqlens[prompt];
   const int len = P.cu_seqlens[prompt + 1] - seq_begin;
-  // Heaviest tiles (most keys) first.
-  const int q0 = (P.q_tiles - 1 - in_group % P.q_tiles) * kBM;
   if (q0 >= len) return;
 
   const int qcol = lane & 31;            // this lane's query column / fragment row
@@ -401,7 +428,8 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
 
 extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const void *q, int64_t q_row_stride,
                                       const void *k, const void *v, int64_t kv_row_stride,
-                                      const int32_t *cu_seqlens, const int32_t *prompt_order, int32_t num_prompts,
+                                      const int32_t *cu_seqlens, const int32_t *prompt_order,
+                                      const int32_t *prompt_lens_host, int32_t num_prompts,
                                       int32_t max_prompt_len, int32_t num_q_heads, int32_t num_kv_heads,
                                       int32_t head_size, float scale, int32_t dtype, void *stream) {
   using namespace mux;
@@ -440,8 +468,27 @@ extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const v
   P.num_groups = num_prompts * num_kv_heads;
   P.scale_log2 = scale * 1.4426950408889634f;
   P.out_rows_16b = (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && out_row_stride % 8 == 0;
-  const int64_t n_wg = static_cast<int64_t>((P.num_groups + 7) / 8) * 8 * P.ratio * P.q_tiles;
-  if (n_wg > 0x7fffffff) return MUXA_EUNSUPPORTED;
+  int64_t n_wg = static_cast<int64_t>((P.num_groups + 7) / 8) * 8 * P.ratio * P.q_tiles;
+  P.n_pairs = 0;
+  P.kv_per_xcd = (num_kv_heads + 7) / 8;
+  if (prompt_lens_host != nullptr && num_prompts <= 0xffff) {
+    // The query tiles that exist, heaviest (most keys) first; ties: as packed.
+    int64_t total = 0;
+    for (int p = 0; p < num_prompts; ++p) {
+      if (prompt_lens_host[p] < 0 || prompt_lens_host[p] > max_prompt_len) return MUXA_EINVAL;
+      total += (prompt_lens_host[p] + kBM - 1) / kBM;
+    }
+    if (total == 0) return MUXA_OK;
+    if (total <= kMaxPairs) {
+      int n = 0;
+      for (int t = P.q_tiles - 1; t >= 0; --t)
+        for (int p = 0; p < num_prompts; ++p)
+          if (t * kBM < prompt_lens_host[p]) P.pairs[n++] = (static_cast<uint32_t>(p) << 16) | static_cast<uint32_t>(t);
+      P.n_pairs = n;
+      n_wg = static_cast<int64_t>(n) * P.kv_per_xcd * P.ratio * 8;
+    }
+  }
+  if (n_wg > 0x7fffffff || P.q_tiles > 0xffff) return MUXA_EUNSUPPORTED;
   const dim3 grid(static_cast<uint32_t>(n_wg));
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == MUXA_DTYPE_F16) hipLaunchKernelGGL((prefill_causal_kernel<F16>), grid, dim3(256), 0, st, P);

@@ -180,10 +180,13 @@ def paged_decode(out, q, k_pool, v_pool, block_tables, context_lens, max_context
 
 
 def prefill_causal(out, q, k, v, cu_seqlens: torch.Tensor, max_prompt_len: int, scale: float,
-                   num_kv_heads: int, stream=None, prompt_order: Optional[torch.Tensor] = None) -> None:
+                   num_kv_heads: int, stream=None, prompt_order: Optional[torch.Tensor] = None,
+                   prompt_lens=None) -> None:
     """Causal attention over packed prompts; cu_seqlens int32 [P+1] on the device.
-    prompt_order: optional int32 [P] on the device, the prompts longest first
-    (scheduling only; results are the same)."""
+    prompt_lens: optional host-side lengths (a sequence of P ints): the launch
+    then holds only the query tiles that exist, heaviest first.  prompt_order:
+    optional int32 [P] on the device, the prompts longest first, used when the
+    lengths are not given.  Scheduling only; results are the same."""
     _need_cuda(out, q, k, v, cu_seqlens)
     order_ptr = None
     if prompt_order is not None:
@@ -201,9 +204,15 @@ def prefill_causal(out, q, k, v, cu_seqlens: torch.Tensor, max_prompt_len: int, 
     kv_stride = _rows(k, "k")
     if _rows(v, "v") != kv_stride:
         raise ValueError("k and v row strides differ")
+    lens_arg = None
+    if prompt_lens is not None:
+        if len(prompt_lens) != cu_seqlens.shape[0] - 1:
+            raise ValueError("prompt_lens: expected one length per prompt")
+        lens_arg = prompt_lens if isinstance(prompt_lens, ctypes.Array) else \
+            (ctypes.c_int32 * len(prompt_lens))(*[int(x) for x in prompt_lens])
     rc = _lib.attn().mux_prefill_causal(
         out.data_ptr(), _rows(out, "out"), q.data_ptr(), _rows(q, "q"), k.data_ptr(), v.data_ptr(), kv_stride,
-        cu_seqlens.data_ptr(), order_ptr, cu_seqlens.shape[0] - 1, int(max_prompt_len), q.shape[1] // HEAD_SIZE,
+        cu_seqlens.data_ptr(), order_ptr, lens_arg, cu_seqlens.shape[0] - 1, int(max_prompt_len), q.shape[1] // HEAD_SIZE,
         int(num_kv_heads), HEAD_SIZE, float(scale), _dtype_code(q), _stream_ptr(stream))
     _lib.check_attn(rc, "mux_prefill_causal")
 

@@ -27,7 +27,7 @@ def _bound(want, dtype):
     return b
 
 
-def _run_prefill(seed, lens, Hq, Hkv, dtype, in_qkv=True):
+def _run_prefill(seed, lens, Hq, Hkv, dtype, in_qkv=True, host_lens=False):
     g = torch.Generator().manual_seed(seed)
     T = int(sum(lens))
     pad = (T + 7) // 8 * 8
@@ -43,7 +43,7 @@ def _run_prefill(seed, lens, Hq, Hkv, dtype, in_qkv=True):
         dq, dk, dv = q.to(DEV), k.to(DEV), v.to(DEV)
     cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32, device=DEV)
     out = torch.full((pad, Hq * D), 7.0, dtype=dtype, device=DEV)
-    ops.prefill_causal(out, dq, dk, dv, cu, int(max(lens)), D ** -0.5, Hkv)
+    ops.prefill_causal(out, dq, dk, dv, cu, int(max(lens)), D ** -0.5, Hkv, prompt_lens=lens if host_lens else None)
     torch.cuda.synchronize()
     got = out.float().cpu()
     assert (got[T:] == 7.0).all(), "padding rows must not be written"
@@ -62,11 +62,13 @@ def test_prefill_matches_oracle_ragged_prompts(Hq, Hkv, dtype):
     assert excess <= 0, f"max-abs error {(got - want).abs().max().item():.3e}"
 
 
+@pytest.mark.parametrize("host_lens", [False, True])
 @pytest.mark.parametrize("num_prompts", [64, 70, 150])
-def test_prefill_many_prompts_ties_and_empty_prompts(num_prompts):
+def test_prefill_many_prompts_ties_and_empty_prompts(num_prompts, host_lens):
     """Many prompts in one launch: equal lengths, empty prompts and lengths
-    around the 128-row tile all appear."""
-    _announce(f"prefill {num_prompts} prompts")
+    around the 128-row tile all appear; with the grid sized by the longest
+    prompt and with the compact grid built from host-side lengths."""
+    _announce(f"prefill {num_prompts} prompts host_lens={host_lens}")
     rng = np.random.Generator(np.random.PCG64(num_prompts))
     lens = rng.integers(1, 200, size=num_prompts)
     lens[::5] = 128
@@ -75,18 +77,19 @@ def test_prefill_many_prompts_ties_and_empty_prompts(num_prompts):
     lens[num_prompts - 2] = 0
     lens[7] = 260
     lens = [int(n) for n in lens]
-    got, q, k, v = _run_prefill(3, lens, 2, 1, torch.float16)
+    got, q, k, v = _run_prefill(3, lens, 2, 1, torch.float16, host_lens=host_lens)
     want = orc.prefill_causal(q, k, v, lens, D ** -0.5, 1)
     assert torch.isfinite(got).all()
     excess = ((got - want).abs() - _bound(want, torch.float16)).max().item()
     assert excess <= 0, f"max-abs error {(got - want).abs().max().item():.3e}"
 
 
+@pytest.mark.parametrize("host_lens", [False, True])
 @pytest.mark.parametrize("Hkv", [5, 9, 13])
-def test_prefill_kv_head_counts_that_do_not_divide_by_eight(Hkv):
-    _announce(f"prefill Hkv={Hkv}")
+def test_prefill_kv_head_counts_that_do_not_divide_by_eight(Hkv, host_lens):
+    _announce(f"prefill Hkv={Hkv} host_lens={host_lens}")
     lens = [130, 17, 64]
-    got, q, k, v = _run_prefill(4, lens, Hkv, Hkv, torch.float16)
+    got, q, k, v = _run_prefill(4, lens, Hkv, Hkv, torch.float16, host_lens=host_lens)
     want = orc.prefill_causal(q, k, v, lens, D ** -0.5, Hkv)
     excess = ((got - want).abs() - _bound(want, torch.float16)).max().item()
     assert excess <= 0, f"max-abs error {(got - want).abs().max().item():.3e}"
@@ -126,6 +129,43 @@ def test_prefill_prompt_order_changes_scheduling_only():
     with pytest.raises(ValueError):
         ops.prefill_causal(base, q, k, v, cu, max(lens), D ** -0.5, 3,
                            prompt_order=torch.zeros((3,), dtype=torch.int32, device=DEV))
+    # the compact grid built from host-side lengths: the same tiles again
+    out = torch.zeros_like(q)
+    ops.prefill_causal(out, q, k, v, cu, max(lens), D ** -0.5, 3, prompt_lens=lens)
+    torch.cuda.synchronize()
+    assert torch.equal(out, base)
+
+
+def test_prefill_host_side_lengths_are_a_hint_not_an_address():
+    """Host-side lengths only choose which query tiles are started: lengths that
+    are too short leave the tiles they hide unwritten, lengths beyond the
+    stated maximum are refused, and a batch with more query tiles than the
+    kernel argument holds falls back to the grid sized by the longest prompt."""
+    _announce("prefill host lengths")
+    lens = [300, 40, 129]
+    T = sum(lens)
+    g = torch.Generator().manual_seed(13)
+    q = torch.randn((T, 2 * D), generator=g).half().to(DEV)
+    k = torch.randn((T, 2 * D), generator=g).half().to(DEV)
+    v = torch.randn((T, 2 * D), generator=g).half().to(DEV)
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32, device=DEV)
+    base = torch.full_like(q, 7.0)
+    ops.prefill_causal(base, q, k, v, cu, 300, D ** -0.5, 2)
+    out = torch.full_like(q, 7.0)
+    ops.prefill_causal(out, q, k, v, cu, 300, D ** -0.5, 2, prompt_lens=[128, 40, 0])
+    torch.cuda.synchronize()
+    started = np.r_[0:128, 300:340]                     # rows of the tiles the short lengths still name
+    hidden = np.r_[128:300, 340:T]
+    assert torch.equal(out[started], base[started]) and (out[hidden] == 7.0).all()
+    with pytest.raises(RuntimeError):
+        ops.prefill_causal(out, q, k, v, cu, 300, D ** -0.5, 2, prompt_lens=[301, 40, 129])
+    with pytest.raises(ValueError):
+        ops.prefill_causal(out, q, k, v, cu, 300, D ** -0.5, 2, prompt_lens=[300, 40])
+    # 1000 prompts of 129 tokens: 2000 query tiles, more than the compact list holds
+    many = [129] * 1000
+    got, q2, k2, v2 = _run_prefill(14, many, 1, 1, torch.float16, host_lens=True)
+    want = orc.prefill_causal(q2, k2, v2, many, D ** -0.5, 1)
+    assert (got - want).abs().max().item() <= TOL
 
 
 def test_prefill_first_token_and_block_diagonal_properties():
@@ -224,7 +264,7 @@ def test_prefill_random_shapes_against_the_oracle(seed):
     lens = [int(x) for x in lens]
     in_qkv = bool(rng.integers(2))
     _announce(f"prefill random seed={seed} Hq={Hkv * ratio} Hkv={Hkv} {dtype} lens={lens} in_qkv={in_qkv}")
-    got, q, k, v = _run_prefill(4000 + seed, lens, Hkv * ratio, Hkv, dtype, in_qkv=in_qkv)
+    got, q, k, v = _run_prefill(4000 + seed, lens, Hkv * ratio, Hkv, dtype, in_qkv=in_qkv, host_lens=bool(seed % 2))
     want = orc.prefill_causal(q, k, v, lens, D ** -0.5, Hkv)
     assert torch.isfinite(got).all()
     excess = ((got - want).abs() - _bound(want, dtype)).max().item()
