@@ -164,7 +164,9 @@ int32_t mux_paged_decode(void *out, int64_t out_row_stride, const void *q, int64
  * only the query tiles that exist, the heaviest of the whole batch first, and
  * prompt_order is not used; batches of more than 896 query tiles of 128 rows
  * fall back to the grid sized by max_prompt_len.  The device-side cu_seqlens
- * stay authoritative for addresses and lengths.  Results depend on neither. */
+ * stay authoritative for addresses and lengths (a host length shorter than the
+ * device's only leaves that prompt's further query tiles unstarted).  With
+ * consistent lengths the results depend on neither. */
 int32_t mux_prefill_causal(void *out, int64_t out_row_stride,
                            const void *q, int64_t q_row_stride,
                            const void *k, const void *v, int64_t kv_row_stride,
