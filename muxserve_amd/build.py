@@ -1,7 +1,8 @@
-"""Compile the two shared libraries of the package, in-tree.
+"""Compile the shared libraries of the package, in-tree.
 
     libmuxhost.so  - g++,   pure host C++ (allocator + batch builder)
     libmuxattn.so  - hipcc, gfx950 kernels + their C ABI
+    libmuxtorch.so - g++,   thin TORCH_LIBRARY operators over libmuxattn.so's C ABI
 
 Run as ``python -m muxserve_amd.build``.  Nothing here runs at import time of
 the package: the loaders in muxserve_amd._lib only open what this step built
@@ -18,6 +19,8 @@ CSRC = os.path.join(PKG, "csrc")
 
 HOST_LIB = os.path.join(PKG, "libmuxhost.so")
 ATTN_LIB = os.path.join(PKG, "libmuxattn.so")
+TORCH_LIB = os.path.join(PKG, "libmuxtorch.so")
+TORCH_SOURCES = [os.path.join(CSRC, "torch", "mux_torch_ops.cpp")]
 
 HOST_SOURCES = [os.path.join(CSRC, "host", f) for f in ("kv_storage.cpp", "batch_scheduler.cpp")]
 HIP_SOURCES = [os.path.join(CSRC, "hip", f) for f in (
@@ -50,11 +53,28 @@ def build_hip(extra=()):
     return ATTN_LIB
 
 
+def build_torch():
+    """The operator library: host C++ only (no device code), linked against
+    torch's libraries and libmuxattn.so next to it."""
+    import torch
+    from torch.utils import cpp_extension
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = ["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-w", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", f"-I{INCLUDE}"]
+    for inc in cpp_extension.include_paths() + ["/opt/rocm/include"]:
+        cmd += ["-isystem", inc]
+    cmd += [*TORCH_SOURCES, "-o", TORCH_LIB, f"-L{tlib}", f"-L{PKG}", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tlib}",
+            "-l:libmuxattn.so", "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip"]
+    _run(cmd)
+    return TORCH_LIB
+
+
 def build_all():
     build_host()
     build_hip()
+    build_torch()
 
 
 if __name__ == "__main__":
     what = sys.argv[1] if len(sys.argv) > 1 else "all"
-    {"host": build_host, "hip": build_hip, "all": build_all}[what]()
+    {"host": build_host, "hip": build_hip, "torch": build_torch, "all": build_all}[what]()

@@ -60,3 +60,17 @@ def test_decode_rejects_malformed_arguments_on_the_host_side():
     rc = lib.mux_reshape_and_cache(16, 16, 128, 16, 16, 8, 16, 0, 1, 4, 1, 64, 16, 0, None)
     assert rc == -2          # head size other than 128
     assert lib.mux_stream_create_cu_range(None, 0, 50, None) == -1
+
+
+def test_torch_operator_library_loads_and_registers_every_operator():
+    """libmuxtorch.so loads without a GPU, registers its operators with the
+    dispatcher, and has no CPU kernels to fall back to."""
+    import pytest
+    import torch
+    from muxserve_amd import torch_ops
+    ns = torch_ops.load()
+    for name in torch_ops.OPERATORS:
+        assert hasattr(ns, name), name
+        assert getattr(ns, name).default._schema.name == f"muxserve_amd::{name}"
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        ns.silu_and_mul(torch.zeros((2, 16), dtype=torch.float16))
