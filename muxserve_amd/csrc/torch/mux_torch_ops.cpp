@@ -12,6 +12,7 @@
 #include <c10/hip/HIPStream.h>
 #include <torch/library.h>
 
+#include <algorithm>
 #include <vector>
 
 #include "muxserve_attn.h"
@@ -174,6 +175,108 @@ void paged_decode(at::Tensor out, const at::Tensor &q, const at::Tensor &k_pool,
         "mux_multi_decode");
 }
 
+// Several colocated models (different head counts, tables, q/out tensors) that
+// share the pool, in one launch: element i of every list describes model i.
+int64_t multi_decode_workspace_bytes(at::TensorList outs, at::TensorList qs, at::TensorList block_tables,
+                                     at::TensorList context_lens, at::IntArrayRef max_context_lens,
+                                     int64_t partition_size) {
+  const size_t n = outs.size();
+  TORCH_CHECK(n >= 1 && n <= MUXA_MAX_DECODE_ITEMS && qs.size() == n && block_tables.size() == n &&
+                  context_lens.size() == n && max_context_lens.size() == n,
+              "multi_decode: 1..", MUXA_MAX_DECODE_ITEMS, " models, one entry per model in every list");
+  MuxDecodeItem items[MUXA_MAX_DECODE_ITEMS];
+  for (size_t i = 0; i < n; ++i)
+    items[i] = decode_item(outs[i], qs[i], block_tables[i], context_lens[i], max_context_lens[i], 1.0, 0, 0);
+  return static_cast<int64_t>(
+      mux_paged_decode_workspace_bytes(items, static_cast<int32_t>(n), static_cast<int32_t>(partition_size)));
+}
+
+void multi_decode(at::TensorList outs, at::TensorList qs, const at::Tensor &k_pool, const at::Tensor &v_pool,
+                  at::TensorList block_tables, at::TensorList context_lens, at::IntArrayRef max_context_lens,
+                  at::ArrayRef<double> scales, at::IntArrayRef layers, at::IntArrayRef total_context_lens,
+                  int64_t partition_size, at::Tensor workspace) {
+  need_gpu({&k_pool, &v_pool});
+  const int64_t bs = check_pools(k_pool, v_pool);
+  const size_t n = outs.size();
+  TORCH_CHECK(n >= 1 && n <= MUXA_MAX_DECODE_ITEMS && qs.size() == n && block_tables.size() == n &&
+                  context_lens.size() == n && max_context_lens.size() == n && scales.size() == n &&
+                  layers.size() == n && total_context_lens.size() == n,
+              "multi_decode: 1..", MUXA_MAX_DECODE_ITEMS, " models, one entry per model in every list");
+  MuxDecodeItem items[MUXA_MAX_DECODE_ITEMS];
+  for (size_t i = 0; i < n; ++i) {
+    TORCH_CHECK(qs[i].scalar_type() == k_pool.scalar_type(), "q dtype must equal the pool dtype");
+    items[i] = decode_item(outs[i], qs[i], block_tables[i], context_lens[i], max_context_lens[i], scales[i],
+                           layers[i], total_context_lens[i]);
+  }
+  void *ws = nullptr;
+  size_t ws_bytes = 0;
+  if (workspace.defined() && workspace.numel() > 0) {
+    TORCH_CHECK(workspace.is_cuda() && workspace.is_contiguous(), "workspace: expected a contiguous GPU tensor");
+    ws = workspace.data_ptr();
+    ws_bytes = static_cast<size_t>(workspace.numel()) * workspace.element_size();
+  }
+  check(mux_multi_decode(items, static_cast<int32_t>(n), k_pool.data_ptr(), v_pool.data_ptr(), k_pool.size(0), kHead,
+                         static_cast<int32_t>(bs), dtype_code(k_pool), static_cast<int32_t>(partition_size), ws,
+                         ws_bytes, stream_of(k_pool)),
+        "mux_multi_decode");
+}
+
+void rotary_neox(const at::Tensor &positions, at::Tensor q, at::Tensor k, const at::Tensor &cos_sin,
+                 int64_t num_tokens) {
+  need_gpu({&positions, &q, &k, &cos_sin});
+  TORCH_CHECK(positions.scalar_type() == at::kLong && positions.dim() == 1 && positions.is_contiguous(),
+              "positions: expected contiguous int64 [T]");
+  TORCH_CHECK(cos_sin.scalar_type() == at::kFloat && cos_sin.dim() == 2 && cos_sin.is_contiguous(),
+              "cos_sin: expected contiguous float32 [max_position, rotary_dim]");
+  TORCH_CHECK(q.dim() == 2 && k.dim() == 2 && q.scalar_type() == k.scalar_type() && q.size(1) % kHead == 0 &&
+                  k.size(1) % kHead == 0,
+              "q [T, Hq*128], k [T, Hkv*128] of one dtype expected");
+  const int64_t T = num_tokens < 0 ? positions.size(0) : num_tokens;
+  TORCH_CHECK(std::min({q.size(0), k.size(0), positions.size(0)}) >= T, "fewer rows than tokens");
+  check(mux_rotary_neox(positions.data_ptr<int64_t>(), q.data_ptr(), rows(q, "q"), k.data_ptr(), rows(k, "k"),
+                        cos_sin.data_ptr<float>(), static_cast<int32_t>(cos_sin.size(0)),
+                        static_cast<int32_t>(cos_sin.size(1)), static_cast<int32_t>(T),
+                        static_cast<int32_t>(q.size(1) / kHead), static_cast<int32_t>(k.size(1) / kHead), kHead,
+                        dtype_code(q), stream_of(q)),
+        "mux_rotary_neox");
+}
+
+// GreedySampler.forward (muxserve/flexserver/sampler.py:15-35) without the
+// logits: int64 [num_rows].  row_index: int32 rows of hidden_states to sample,
+// or an empty tensor for rows 0 .. num_rows-1.  workspace: uint8,
+// greedy_sample_workspace_bytes(vocab_size) bytes, zero-filled before its first
+// use (every call leaves its counter zero).
+int64_t greedy_sample_workspace_bytes(int64_t vocab_size) {
+  return static_cast<int64_t>(mux_greedy_sample_workspace_bytes(static_cast<int32_t>(vocab_size)));
+}
+
+at::Tensor greedy_sample(const at::Tensor &embedding, const at::Tensor &hidden_states, int64_t vocab_size,
+                         int64_t num_rows, const at::Tensor &row_index, at::Tensor workspace) {
+  need_gpu({&embedding, &hidden_states, &workspace});
+  TORCH_CHECK(embedding.dim() == 2 && hidden_states.dim() == 2 && embedding.size(1) == hidden_states.size(1) &&
+                  embedding.scalar_type() == hidden_states.scalar_type(),
+              "embedding [V, hidden] and hidden_states [T, hidden] of one dtype expected");
+  const int32_t *ri = nullptr;
+  if (row_index.defined() && row_index.numel() > 0) {
+    TORCH_CHECK(row_index.is_cuda() && row_index.scalar_type() == at::kInt && row_index.dim() == 1 &&
+                    row_index.is_contiguous() && row_index.size(0) >= num_rows,
+                "row_index: expected contiguous int32 [>= num_rows] on the GPU");
+    ri = row_index.data_ptr<int32_t>();
+  } else {
+    TORCH_CHECK(hidden_states.size(0) >= num_rows, "fewer rows of hidden states than sampled rows");
+  }
+  TORCH_CHECK(workspace.is_contiguous(), "workspace: expected a contiguous GPU tensor");
+  at::Tensor out = at::empty({num_rows}, hidden_states.options().dtype(at::kLong));
+  check(mux_greedy_sample(out.data_ptr<int64_t>(), hidden_states.data_ptr(), rows(hidden_states, "hidden_states"),
+                          static_cast<int32_t>(hidden_states.size(0)), ri, static_cast<int32_t>(num_rows),
+                          embedding.data_ptr(), rows(embedding, "embedding"), static_cast<int32_t>(embedding.size(0)),
+                          static_cast<int32_t>(vocab_size), static_cast<int32_t>(hidden_states.size(1)),
+                          dtype_code(hidden_states), workspace.data_ptr(),
+                          static_cast<size_t>(workspace.numel()) * workspace.element_size(), stream_of(hidden_states)),
+        "mux_greedy_sample");
+  return out;
+}
+
 void prefill_causal(at::Tensor out, const at::Tensor &q, const at::Tensor &k, const at::Tensor &v,
                     const at::Tensor &cu_seqlens, at::IntArrayRef prompt_lens, int64_t max_prompt_len, double scale,
                     int64_t num_kv_heads) {
@@ -242,6 +345,15 @@ TORCH_LIBRARY(muxserve_amd, m) {
         "int total_context_len, Tensor(b!) workspace) -> ()");
   m.def("prefill_causal(Tensor(a!) out, Tensor q, Tensor k, Tensor v, Tensor cu_seqlens, int[] prompt_lens, "
         "int max_prompt_len, float scale, int num_kv_heads) -> ()");
+  m.def("multi_decode_workspace_bytes(Tensor[] outs, Tensor[] qs, Tensor[] block_tables, Tensor[] context_lens, "
+        "int[] max_context_lens, int partition_size) -> int");
+  m.def("multi_decode(Tensor(a!)[] outs, Tensor[] qs, Tensor k_pool, Tensor v_pool, Tensor[] block_tables, "
+        "Tensor[] context_lens, int[] max_context_lens, float[] scales, int[] layers, int[] total_context_lens, "
+        "int partition_size, Tensor(b!) workspace) -> ()");
+  m.def("rotary_neox(Tensor positions, Tensor(a!) q, Tensor(b!) k, Tensor cos_sin, int num_tokens) -> ()");
+  m.def("greedy_sample_workspace_bytes(int vocab_size) -> int", &greedy_sample_workspace_bytes);
+  m.def("greedy_sample(Tensor embedding, Tensor hidden_states, int vocab_size, int num_rows, Tensor row_index, "
+        "Tensor(a!) workspace) -> Tensor");
   m.def("rms_norm(Tensor x, Tensor weight, float eps) -> Tensor");
   m.def("silu_and_mul(Tensor x) -> Tensor");
 }
@@ -252,6 +364,10 @@ TORCH_LIBRARY_IMPL(muxserve_amd, CUDA, m) {
   m.impl("paged_decode_workspace_bytes", &paged_decode_workspace_bytes);
   m.impl("paged_decode", &paged_decode);
   m.impl("prefill_causal", &prefill_causal);
+  m.impl("multi_decode_workspace_bytes", &multi_decode_workspace_bytes);
+  m.impl("multi_decode", &multi_decode);
+  m.impl("rotary_neox", &rotary_neox);
+  m.impl("greedy_sample", &greedy_sample);
   m.impl("rms_norm", &rms_norm);
   m.impl("silu_and_mul", &silu_and_mul);
 }

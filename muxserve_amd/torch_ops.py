@@ -20,8 +20,9 @@ from ._lib import MuxLibraryMissing
 _PKG = os.path.dirname(os.path.abspath(__file__))
 TORCH_LIB_PATH = os.environ.get("MUXSERVE_TORCH_LIB", os.path.join(_PKG, "libmuxtorch.so"))
 
-OPERATORS = ("reshape_and_cache", "rope_reshape_and_cache", "paged_decode_workspace_bytes", "paged_decode",
-             "prefill_causal", "rms_norm", "silu_and_mul")
+OPERATORS = ("reshape_and_cache", "rope_reshape_and_cache", "rotary_neox", "paged_decode_workspace_bytes",
+             "paged_decode", "multi_decode_workspace_bytes", "multi_decode", "prefill_causal", "rms_norm",
+             "silu_and_mul", "greedy_sample_workspace_bytes", "greedy_sample")
 
 _loaded = False
 

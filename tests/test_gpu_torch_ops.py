@@ -80,6 +80,32 @@ def test_torch_operators_equal_the_ctypes_path(dtype):
         T.paged_decode(o2, dq, k_pool, v_pool, d_bt, d_ctx, int(ctx.max()), D ** -0.5, 1, 64, 0, ws)
     torch.cuda.synchronize()
     assert torch.equal(_bits(o1), _bits(o2)) and o1[:3].float().abs().sum().item() > 0
+    # ---- the fused launch over two "models" (the same tables twice, different queries) -----
+    dq2 = torch.randn((8, Hq * D), generator=g).to(dtype).to(DEV)
+    f1, f2 = torch.zeros_like(o1), torch.zeros_like(o1)
+    lists = ([f1, f2], [dq, dq2], [d_bt, d_bt], [d_ctx, d_ctx], [int(ctx.max())] * 2)
+    need2 = T.multi_decode_workspace_bytes(*lists, 64)
+    ws2 = torch.zeros((need2,), dtype=torch.uint8, device=DEV)
+    T.multi_decode(lists[0], lists[1], k_pool, v_pool, lists[2], lists[3], lists[4], [D ** -0.5] * 2, [1, 1],
+                   [int(ctx.sum())] * 2, 64, ws2)
+    o3 = torch.zeros_like(o1)
+    ops.paged_decode(o3, dq2, k_pool, v_pool, d_bt, d_ctx, int(ctx.max()), D ** -0.5, layer=1, partition_size=64)
+    torch.cuda.synchronize()
+    assert torch.equal(_bits(f1), _bits(o1)) and torch.equal(_bits(f2), _bits(o3))
+    # ---- stand-alone rotary, greedy sampling ---------------------------------------------
+    r1 = qkv.clone().split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+    r2 = qkv.clone().split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+    ops.rotary_neox(positions, r1[0], r1[1], cos_sin, num_tokens=n)
+    T.rotary_neox(positions, r2[0], r2[1], cos_sin, n)
+    assert torch.equal(_bits(r1[0]), _bits(r2[0])) and torch.equal(_bits(r1[1]), _bits(r2[1]))
+    V = 1000
+    emb = (torch.randn((V + 8, 512), generator=g) * 0.1).to(dtype).to(DEV)
+    hid = torch.randn((12, 512), generator=g).to(dtype).to(DEV)
+    ri = torch.tensor([11, 0, 5], dtype=torch.int32, device=DEV)
+    wss = torch.zeros((T.greedy_sample_workspace_bytes(V),), dtype=torch.uint8, device=DEV)
+    none = torch.empty((0,), dtype=torch.int32, device=DEV)
+    assert torch.equal(T.greedy_sample(emb, hid, V, 3, ri, wss), ops.greedy_sample(emb, hid, V, 3, row_index=ri))
+    assert torch.equal(T.greedy_sample(emb, hid, V, 12, none, wss), ops.greedy_sample(emb, hid, V, 12))
     # ---- layer operators -----------------------------------------------------------------
     x = (torch.randn((9, 1024), generator=g) * 2).to(dtype).to(DEV)
     w = (1 + 0.1 * torch.randn((1024,), generator=g)).to(dtype).to(DEV)
