@@ -26,3 +26,19 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def _return_large_pools_to_the_device(request):
+    """The full-size pool tests allocate 185 GB and 200 GB.  Left in torch's
+    caching allocator, the first pool makes the next test's allocation fail in
+    the driver and succeed only on the allocator's free-everything-and-retry
+    path; a test run has crashed inside that path (host segmentation fault in
+    torch.empty).  Large caches are therefore handed back after every GPU test,
+    so that no allocation is ever made on the edge of the device's memory."""
+    yield
+    if "gpu" in request.keywords:
+        import torch
+        if torch.cuda.is_available() and torch.cuda.memory_reserved() > (16 << 30):
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
