@@ -327,13 +327,21 @@ def bench_gqa_long(args):
     ms = _time(step, args.steps, args.warmup)
     nbytes = float(np.mean([workloads.decode_bytes(m.context_lens, 64, 8, bs) for m in sets]))
     gbs = nbytes / (ms * 1e-3) / 1e9
+    # The yardstick: the same blocks read by the bare gather-read probe.
+    used = [torch.from_numpy(m.used_blocks(bs).astype(np.int32)).to(dev) for m in sets]
+    sink = torch.zeros((1,), dtype=torch.int32, device=dev)
+    probe_ms = _time(lambda i: ops.probe_gather_read(k_pool, v_pool, used[i % len(used)], sink), args.steps, args.warmup)
+    probe_bytes = float(np.mean([u.numel() * 8192 for u in used]))
     cfg = {"workload": "gqa_long", "shape": "Hq64/Hkv8, B=64, ctx U[2048,8192], bf16", "pool_gb": round(N * 8192 / 1e9, 1),
            "bytes_per_step": int(nbytes), "partition": args.partition}
     roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
             "traffic": nbytes * GQA_LONG_TRAFFIC_RATIO,
             "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
                               "profiles/paged_decode_gqa_long_kernel_trace_and_traffic.txt",
-            "kernel": "paged_decode_gqa_kernel<BF16,16,8,4>"}
+            "kernel": "paged_decode_gqa_kernel<BF16,16,8,4>",
+            "bare_gather_read_of_the_same_blocks": {
+                "ms": probe_ms, "bytes": int(probe_bytes), "GB/s": probe_bytes / (probe_ms * 1e-3) / 1e9,
+                "kernel": "probe_gather_read_kernel (whole 4 KiB blocks, no arithmetic)"}}
     return _line("long-context GQA decode attn tokens/s", 64 / (ms * 1e-3), "tokens/s", args, ms, cfg, roof, dtype="bf16")
 
 
