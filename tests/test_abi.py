@@ -74,3 +74,14 @@ def test_torch_operator_library_loads_and_registers_every_operator():
         assert getattr(ns, name).default._schema.name == f"muxserve_amd::{name}"
     with pytest.raises((NotImplementedError, RuntimeError)):
         ns.silu_and_mul(torch.zeros((2, 16), dtype=torch.float16))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py is a one-GPU benchmark: --gpus N > 1 exits with a message
+    before anything touches a device."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout.strip() == ""
