@@ -125,6 +125,16 @@ __device__ __forceinline__ float wave_sum(float v) {
   return (lane_bcast(v, 0) + lane_bcast(v, 16)) + (lane_bcast(v, 32) + lane_bcast(v, 48));
 }
 
+// Blocks this wave until every vector-memory access it has issued - loads AND
+// stores - has completed (on gfx9 stores count in vmcnt and are acknowledged
+// once they have reached the level their scope bits name).  A workgroup-scope
+// fence does not emit this wait for agent-scope relaxed stores, so code that
+// publishes data to other workgroups and then bumps an arrival counter calls it
+// between the two.
+__device__ __forceinline__ void wait_own_vector_memory() {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Inclusive prefix sum over the 64 lanes of a wave (row shifts, then the two

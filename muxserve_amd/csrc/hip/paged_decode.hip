@@ -343,11 +343,14 @@ __device__ __forceinline__ void merge_and_write(const DecodeItemDev &I, const Un
   if (single) return;
 
   // Partials are written and read with device-coherent accesses (they bypass
-  // the per-XCD L2), so ordering them against the arrival counter needs only
-  // "my stores have completed" / "my loads issue after the atomic returned" -
-  // a workgroup-scope fence, i.e. a wait, not an L2 write-back/invalidate.
+  // the per-XCD L2 and are acknowledged from the memory side), so ordering them
+  // against the arrival counter needs no L2 write-back/invalidate, only: (1) this
+  // wave's partial stores have been acknowledged before the counter is bumped -
+  // the explicit vmcnt wait; (2) the combiner's loads issue after its atomic
+  // returned - they depend on its value.  The fences only pin the compiler.
   const int n_splits = (u.ctx + partition - 1) / partition;
   int32_t *counter = I.counters + static_cast<int64_t>(u.seq) * (I.Hq / G) + u.wh;
+  wait_own_vector_memory();
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   int arrived = 0;
   if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -403,11 +406,13 @@ __device__ __forceinline__ void merge_and_write_group(const DecodeItemDev &I, co
   }
   if (single) return;
 
-  // Each wave waits for its own partial stores (they bypass the per-XCD L2, so
-  // completion is all that is needed), the workgroup meets, one lane announces
-  // the arrival and tells the others whether this workgroup came last.
+  // Each wave waits until its own partial stores have been acknowledged (they
+  // bypass the per-XCD L2, so the acknowledgement is all that is needed), the
+  // workgroup meets, one lane announces the arrival and tells the others
+  // whether this workgroup came last.
   const int n_splits = (u.ctx + partition - 1) / partition;
   int32_t *counter = I.counters + static_cast<int64_t>(u.seq) * (I.Hq / G) + u.wh;
+  wait_own_vector_memory();
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (wave == 0 && lane == 0)

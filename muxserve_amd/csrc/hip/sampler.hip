@@ -263,10 +263,12 @@ __global__ __launch_bounds__(64 * NW) void lm_head_argmax_kernel(const LmHeadPar
                        __HIP_MEMORY_SCOPE_AGENT);
   }
   // The table is written and read with device-coherent accesses (they bypass
-  // the per-XCD L2), so ordering them against the counter takes only a
-  // workgroup-scope fence, i.e. a wait.  A device-scope fence would write back
-  // and invalidate this XCD's L2, which holds the hidden states every other
+  // the per-XCD L2), so ordering them against the counter takes only a wait
+  // for this wave's table stores to be acknowledged before the workgroup meets
+  // and bumps the counter.  A device-scope fence would also write back and
+  // invalidate this XCD's L2, which holds the hidden states every other
   // workgroup is still reading (measured: +30 us per launch).
+  wait_own_vector_memory();
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (tid == 0)
