@@ -46,6 +46,8 @@ extern "C" {
 #define MUXA_EUNSUPPORTED (-2)/* head size != 128, block size not 8/16/32 ...  */
 #define MUXA_EWORKSPACE (-3)  /* workspace missing or too small                */
 #define MUXA_EHIP (-4)        /* a HIP runtime call failed (see mux_last_hip_error) */
+#define MUXA_ESCRATCH_LIMIT (-5) /* the call needs more scratch than the library's fixed
+                                    static array holds (mux_multi_decode_noalloc only)  */
 
 #define MUXA_DTYPE_F16 0
 #define MUXA_DTYPE_BF16 1
@@ -137,6 +139,28 @@ int32_t mux_multi_decode(const MuxDecodeItem *items, int32_t n_items,
                          int32_t head_size, int32_t block_size, int32_t dtype,
                          int32_t partition_size, void *workspace, size_t workspace_bytes,
                          void *stream);
+
+/* mux_multi_decode for callers that cannot allocate.  No counterpart in the
+ * reference: it exists for callers that must not call hipMalloc or any
+ * allocating routine - code under HIP graph capture, tight serving loops,
+ * harnesses that forbid it - and that have no workspace of their own to pass.
+ * Same arguments, results and kernels as mux_multi_decode, except that the
+ * scratch (arrival counters, partial results of split contexts, the pair table
+ * of large batches) is a static device array of MUXA_STATIC_SCRATCH_BYTES inside
+ * the library: one copy per GPU the library runs on, held until the process
+ * ends.  The call allocates and frees nothing, records no memset (its arrival
+ * counters are cleared by a small fill kernel on `stream` ahead of the
+ * attention kernel) and never synchronises.  A call whose scratch need
+ * (mux_paged_decode_workspace_bytes) exceeds MUXA_STATIC_SCRATCH_BYTES is
+ * refused with MUXA_ESCRATCH_LIMIT before anything is launched.  Every call on
+ * a GPU shares that GPU's array: calls that overlap in time on one GPU (two
+ * streams, two threads) race on it and must be serialised by the caller. */
+#define MUXA_STATIC_SCRATCH_BYTES (32u << 20)
+size_t mux_multi_decode_noalloc_max_bytes(void);
+int32_t mux_multi_decode_noalloc(const MuxDecodeItem *items, int32_t n_items,
+                                 const void *k_pool, const void *v_pool, int64_t num_pool_blocks,
+                                 int32_t head_size, int32_t block_size, int32_t dtype,
+                                 int32_t partition_size, void *stream);
 
 /* Single-model convenience wrapper around mux_multi_decode. */
 int32_t mux_paged_decode(void *out, int64_t out_row_stride, const void *q, int64_t q_row_stride,

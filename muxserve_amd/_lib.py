@@ -123,6 +123,8 @@ ATTN_SIGNATURES = {
     "mux_paged_decode_workspace_init": (c_i32, [c_vp, c_sz, c_vp]),
     "mux_multi_decode": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_i32,
                                  c_vp, c_sz, c_vp]),
+    "mux_multi_decode_noalloc_max_bytes": (c_sz, []),
+    "mux_multi_decode_noalloc": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_i32, c_vp]),
     "mux_paged_decode": (c_i32, [c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_vp,
                                  c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32,
                                  c_f32, c_i32, c_i32, c_vp, c_sz, c_vp]),
@@ -162,7 +164,8 @@ def attn():
 
 
 ATTN_ERRORS = {-1: "invalid argument", -2: "unsupported shape or dtype",
-               -3: "workspace missing or too small", -4: "HIP runtime error"}
+               -3: "workspace missing or too small", -4: "HIP runtime error",
+               -5: "the call needs more scratch than the library's fixed static array holds"}
 
 
 def check_attn(rc, what):

@@ -35,6 +35,7 @@
 #include "mux_common.h"
 
 #include <algorithm>
+#include <mutex>
 
 namespace mux {
 
@@ -1143,12 +1144,16 @@ int32_t mux_paged_decode_workspace_init(void *workspace, size_t workspace_bytes,
   return MUXA_OK;
 }
 
-int32_t mux_multi_decode(const MuxDecodeItem *items, int32_t n_items,
-                         const void *k_pool, const void *v_pool, int64_t num_pool_blocks,
-                         int32_t head_size, int32_t block_size, int32_t dtype,
-                         int32_t partition_size, void *workspace, size_t workspace_bytes,
-                         void *stream) {
-  using namespace mux;
+}  // extern "C"
+
+namespace mux {
+namespace {
+
+int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
+                          const void *k_pool, const void *v_pool, int64_t num_pool_blocks,
+                          int32_t head_size, int32_t block_size, int32_t dtype,
+                          int32_t partition_size, void *workspace, size_t workspace_bytes,
+                          void *stream) {
   if (!items || n_items <= 0 || n_items > MUXA_MAX_DECODE_ITEMS) return MUXA_EINVAL;
   if (!k_pool || !v_pool || num_pool_blocks <= 0) return MUXA_EINVAL;
   if ((reinterpret_cast<uintptr_t>(k_pool) & 15u) || (reinterpret_cast<uintptr_t>(v_pool) & 15u))
@@ -1238,6 +1243,88 @@ int32_t mux_multi_decode(const MuxDecodeItem *items, int32_t n_items,
     if (e != hipSuccess) return hip_fail(e);
   }
   return MUXA_OK;
+}
+
+}  // namespace
+}  // namespace mux
+
+// Scratch of the allocation-free entry point: one copy per GPU the library's
+// code object is loaded on, held until the process ends.  Host code must not
+// use this name as an address; it asks the runtime for the device address once
+// per device (static_scratch_base) and passes that pointer on.
+static __device__ __align__(256) unsigned char scratch[MUXA_STATIC_SCRATCH_BYTES];
+
+namespace mux {
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// Device address of `scratch` on the current device, looked up on the first
+// call per device.  Returns MUXA_OK and sets *out, or a negative code.
+int32_t static_scratch_base(void **out) {
+  int dev = -1;
+  MUX_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return MUXA_EUNSUPPORTED;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *ptr = nullptr;
+    MUX_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) return MUXA_EHIP;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return MUXA_OK;
+}
+
+}  // namespace
+}  // namespace mux
+
+extern "C" {
+
+int32_t mux_multi_decode(const MuxDecodeItem *items, int32_t n_items,
+                         const void *k_pool, const void *v_pool, int64_t num_pool_blocks,
+                         int32_t head_size, int32_t block_size, int32_t dtype,
+                         int32_t partition_size, void *workspace, size_t workspace_bytes,
+                         void *stream) {
+  return mux::multi_decode_impl(items, n_items, k_pool, v_pool, num_pool_blocks, head_size, block_size, dtype,
+                                partition_size, workspace, workspace_bytes, stream);
+}
+
+size_t mux_multi_decode_noalloc_max_bytes(void) { return MUXA_STATIC_SCRATCH_BYTES; }
+
+int32_t mux_multi_decode_noalloc(const MuxDecodeItem *items, int32_t n_items,
+                                 const void *k_pool, const void *v_pool, int64_t num_pool_blocks,
+                                 int32_t head_size, int32_t block_size, int32_t dtype,
+                                 int32_t partition_size, void *stream) {
+  using namespace mux;
+  if (!items || n_items <= 0 || n_items > MUXA_MAX_DECODE_ITEMS) return MUXA_EINVAL;
+  if (partition_size < 0 || partition_size % 64 != 0) return MUXA_EINVAL;
+  for (int i = 0; i < n_items; ++i)
+    if (items[i].num_kv_heads <= 0 || items[i].num_q_heads <= 0 || items[i].num_seqs < 0 ||
+        items[i].max_context_len < 0 || items[i].total_context_len < 0)
+      return MUXA_EINVAL;
+  // The call's scratch need against the fixed size of the static array.
+  const int partition = choose_partition(items, n_items, partition_size);
+  const size_t need = plan_workspace(items, n_items, partition, nullptr);
+  if (need == SIZE_MAX) return MUXA_EUNSUPPORTED;
+  if (need > MUXA_STATIC_SCRATCH_BYTES) return MUXA_ESCRATCH_LIMIT;
+  void *base = nullptr;
+  const int32_t rc = static_scratch_base(&base);
+  if (rc != MUXA_OK) return rc;
+  if (need > 0) {
+    // The array keeps the previous call's contents.  Partials and the pair
+    // table are written before they are read; the arrival counters must start
+    // at zero and every completed launch leaves them so, but a launch that was
+    // cut short would not - so they are cleared here, with a fill kernel (a
+    // memset node must not end up in a captured graph).
+    const int32_t irc = mux_paged_decode_workspace_init(base, MUXA_DECODE_COUNTER_BYTES, stream);
+    if (irc != MUXA_OK) return irc;
+  }
+  return multi_decode_impl(items, n_items, k_pool, v_pool, num_pool_blocks, head_size, block_size, dtype,
+                           partition_size, need > 0 ? base : nullptr, need > 0 ? MUXA_STATIC_SCRATCH_BYTES : 0,
+                           stream);
 }
 
 int32_t mux_paged_decode(void *out, int64_t out_row_stride, const void *q, int64_t q_row_stride,

@@ -171,6 +171,25 @@ def multi_decode(calls: List[DecodeCall], k_pool: torch.Tensor, v_pool: torch.Te
     _lib.check_attn(rc, "mux_multi_decode")
 
 
+def multi_decode_noalloc(calls: List[DecodeCall], k_pool: torch.Tensor, v_pool: torch.Tensor,
+                         partition_size: int = 0, stream=None) -> None:
+    """multi_decode through the entry point that allocates nothing: scratch is
+    the library's static per-GPU array (a fixed 32 MiB; larger needs raise).
+    Calls that overlap in time on one GPU race on that array."""
+    if not 1 <= len(calls) <= _lib.MUXA_MAX_DECODE_ITEMS:
+        raise ValueError(f"1..{_lib.MUXA_MAX_DECODE_ITEMS} models per launch")
+    _need_cuda(k_pool, v_pool)
+    bs = _check_pools(k_pool, v_pool)
+    items = (_lib.MuxDecodeItem * len(calls))(*[c.to_item() for c in calls])
+    for c in calls:
+        if c.q.dtype != k_pool.dtype:
+            raise TypeError("q dtype must equal the pool dtype")
+    rc = _lib.attn().mux_multi_decode_noalloc(ctypes.addressof(items), len(calls), k_pool.data_ptr(),
+                                              v_pool.data_ptr(), k_pool.shape[0], HEAD_SIZE, bs,
+                                              _dtype_code(k_pool), int(partition_size), _stream_ptr(stream))
+    _lib.check_attn(rc, "mux_multi_decode_noalloc")
+
+
 def paged_decode(out, q, k_pool, v_pool, block_tables, context_lens, max_context_len, scale,
                  layer: int = 0, partition_size: int = 0, workspace=None, stream=None,
                  total_context_len: int = 0) -> None:
