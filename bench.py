@@ -52,6 +52,8 @@ def parse():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-hint", action="store_true", help="do not pass the host-side sum of context lengths")
+    ap.add_argument("--no-host-lens", action="store_true",
+                    help="do not pass the host copy of the context lengths (units are then enumerated on the device)")
     ap.add_argument("--no-prompt-order", action="store_true",
                     help="prefill3: start the prompts' workgroups as packed instead of longest first")
     ap.add_argument("--no-prompt-lens", action="store_true",
@@ -606,7 +608,9 @@ def main():
         for j, m in enumerate(models):
             m.to_device(dev, torch.float16, seed=args.seed + 1000 + 10 * i + j)
         calls = [ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
-                                total_context_len=0 if args.no_hint else int(m.context_lens.sum()))
+                                total_context_len=0 if args.no_hint else int(m.context_lens.sum()),
+                                context_lens_host=None if (args.no_hint or args.no_host_lens)
+                                else torch.from_numpy(np.ascontiguousarray(m.context_lens, dtype=np.int32)))
                  for m in models]
         sets.append((models, calls, torch.from_numpy(used.astype(np.int32)).to(dev)))
     torch.cuda.synchronize()

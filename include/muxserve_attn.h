@@ -95,6 +95,16 @@ int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t kv_row_strid
  * total_context_len: optional host-side upper bound on the sum of
  * context_lens (the serving loop has them on the host before the copy,
  * llm_runtime.py:311-326); it only tightens the grid, 0 = unknown.
+ * context_lens_host: optional HOST copy of context_lens [num_seqs] (same
+ * place in the serving loop, llm_runtime.py:311-326: the lengths are a host
+ * list before they become a tensor).  When every model of a launch comes with
+ * one and the batch is small (at most 384 (sequence, partition) pairs), the
+ * work list is enumerated on the host and travels in the kernel argument, so a
+ * workgroup reaches its K/V loads one dependent memory latency sooner.  The
+ * launch then follows the HOST values (clamped to max_context_len) and does not
+ * read the device tensor: they must be equal.  The values are fixed when the
+ * call is made, so leave this NULL for launches recorded into a HIP graph that
+ * is replayed with changed lengths.  NULL = enumerate on the device.
  * partition_size: tokens per split of a context (multiple of 64), 0 = choose.
  * workspace: scratch for the partial results of split contexts and, for
  * batches of more than 256 sequences, the table that maps workgroups to
@@ -122,6 +132,7 @@ typedef struct MuxDecodeItem {
   int32_t max_blocks;
   int32_t max_context_len;
   float scale;
+  const int32_t *context_lens_host; /* optional HOST copy of context_lens, or NULL (see above) */
 } MuxDecodeItem;
 
 size_t mux_paged_decode_workspace_bytes(const MuxDecodeItem *items, int32_t n_items,

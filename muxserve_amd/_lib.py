@@ -111,6 +111,7 @@ class MuxDecodeItem(ctypes.Structure):
         ("num_q_heads", c_i32), ("num_kv_heads", c_i32),
         ("max_blocks", c_i32), ("max_context_len", c_i32),
         ("scale", c_f32),
+        ("context_lens_host", c_vp),
     ]
 
 

@@ -43,6 +43,11 @@ class InputMetadata:
     # Not in the reference: host-side sum of context_lens, if the caller has it
     # (prepare_inputs does); only tightens the decode grid.
     total_context_len: int = 0
+    # Not in the reference either: a host copy of context_lens (CPU int32 [B];
+    # the serving loop has the lengths on the host before they become a tensor,
+    # llm_runtime.py:311-326).  Small decode batches are then enumerated on the
+    # host.  Leave None when the step is recorded into a HIP graph.
+    context_lens_host: Optional[torch.Tensor] = None
     is_muxserve: bool = True                   # read at models/llama.py:285
     _cu_seqlens: Optional[torch.Tensor] = field(default=None, repr=False)
     _prompt_order: Optional[torch.Tensor] = field(default=None, repr=False)
@@ -161,7 +166,8 @@ class PagedAttention(torch.nn.Module):
                 raise ValueError("decode needs the KV pool")
             ops.paged_decode(out[n_prompt:n_valid], query[n_prompt:n_valid], key_cache, value_cache,
                              md.block_tables, md.context_lens, md.max_context_len, self.scale, layer=layer,
-                             partition_size=self.partition_size, total_context_len=md.total_context_len)
+                             partition_size=self.partition_size, total_context_len=md.total_context_len,
+                             context_lens_host=md.context_lens_host)
         return out
 
 

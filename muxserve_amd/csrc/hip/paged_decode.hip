@@ -56,8 +56,16 @@ struct DecodeItemDev {
   int32_t B, Hq, Hkv, ratio;      // ratio = Hq / Hkv
   int32_t max_blocks, max_splits, max_ctx;
   int32_t work_begin;             // first block of this item in the grid
+  int32_t pair_begin;             // first entry of this item in DecodeParams::pairs (host-enumerated launches)
   float scale_log2;               // scale * log2(e)
 };
+
+// Launches whose context lengths the caller also has on the host carry their
+// (sequence, partition) pairs in the kernel argument itself: a workgroup then
+// knows its unit after scalar loads from the (cached) argument segment instead
+// of a round of vector loads of the device-side context lengths - one
+// dependent memory latency less before its K/V loads go out.
+constexpr int kMaxHostPairs = 384;
 
 struct DecodeParams {
   DecodeItemDev it[MUXA_MAX_DECODE_ITEMS];
@@ -66,7 +74,10 @@ struct DecodeParams {
   int32_t n_items;
   int32_t partition;
   int32_t last_block;             // num_pool_blocks - 1: table entries are clamped to it
+  int32_t n_host_pairs;           // > 0: units come from `pairs`, the device-side context lengths are not read
+  uint2 pairs[kMaxHostPairs];     // x = sequence | partition index << 16, y = clamped context length
 };
+static_assert(sizeof(DecodeParams) <= 4096, "kernel argument segment");
 
 // One unit of work, uniform across the workgroup.
 struct Unit {
@@ -518,8 +529,16 @@ __device__ __forceinline__ bool locate_pair_small(const int32_t *ctx_arr, int B,
 
 // Batches too large for that take the pair from a table that a small kernel
 // (decode_plan_kernel below) writes ahead of the launch: one 16-byte load.
-__device__ __forceinline__ bool locate_pair(const DecodeItemDev &I, int partition, int e, int lane, int &seq,
-                                            int &split, int &ctx) {
+__device__ __forceinline__ bool locate_pair(const DecodeParams &P, const DecodeItemDev &I, int partition, int e,
+                                            int lane, int &seq, int &split, int &ctx) {
+  if (P.n_host_pairs > 0) {
+    // The grid of such a launch holds exactly the enumerated pairs.
+    const uint2 pr = P.pairs[min(I.pair_begin + e, kMaxHostPairs - 1)];
+    seq = static_cast<int>(pr.x & 0xffffu);
+    split = static_cast<int>(pr.x >> 16);
+    ctx = static_cast<int>(pr.y);
+    return true;
+  }
   if (I.unit_table == nullptr) return locate_pair_small(I.ctx, I.B, I.max_ctx, partition, e, lane, seq, split, ctx);
   const int4 ent = I.unit_table[e];
   if (ent.x < 0) return false;
@@ -635,7 +654,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_kernel(const DecodeParam
   u.wh = local - e * WH;
   const int partition = P.partition;
   // Every wave of the workgroup derives the same unit (or all of them leave).
-  if (!locate_pair(I, partition, e, lane, u.seq, u.split, u.ctx)) return;
+  if (!locate_pair(P, I, partition, e, lane, u.seq, u.split, u.ctx)) return;
   u.t0 = u.split * partition;
   u.t1 = min(u.ctx, u.t0 + partition);
   const int hq0 = u.wh * G;
@@ -769,7 +788,7 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
   u.item = ii;
   u.wh = local - e * WH;
   const int partition = P.partition;
-  if (!locate_pair(I, partition, e, lane, u.seq, u.split, u.ctx)) return;
+  if (!locate_pair(P, I, partition, e, lane, u.seq, u.split, u.ctx)) return;
   u.t0 = u.split * partition;
   u.t1 = min(u.ctx, u.t0 + partition);
   const int hq0 = u.wh * G;
@@ -1064,6 +1083,38 @@ size_t plan_workspace(const MuxDecodeItem *items, int n_items, int partition, It
   return off;
 }
 
+// Host-side enumeration of one item's (sequence, partition) pairs, in the
+// order the device-side enumeration (locate_pair_small) uses: remainders of
+// split sequences, their full partitions, then the sequences that fit one
+// partition.  Appends to out[*n]; false when they do not fit the kernel
+// argument's table or its 16-bit fields.
+bool enumerate_pairs_on_host(const int32_t *ctx_host, int B, int max_ctx, int partition, uint2 *out, int *n) {
+  if (B > 0xffff) return false;
+  auto clamped = [&](int s) { return std::max(std::min(ctx_host[s], max_ctx), 0); };
+  int at = *n;
+  auto push = [&](int s, int split, int c) {
+    if (at >= kMaxHostPairs || split > 0xffff) return false;
+    out[at++] = make_uint2(static_cast<uint32_t>(s) | (static_cast<uint32_t>(split) << 16), static_cast<uint32_t>(c));
+    return true;
+  };
+  for (int s = 0; s < B; ++s) {
+    const int c = clamped(s), q = c / partition;
+    if (c > partition && c != q * partition && !push(s, q, c)) return false;
+  }
+  for (int s = 0; s < B; ++s) {
+    const int c = clamped(s), q = c / partition;
+    if (c > partition)
+      for (int j = 0; j < q; ++j)
+        if (!push(s, j, c)) return false;
+  }
+  for (int s = 0; s < B; ++s) {
+    const int c = clamped(s);
+    if (c > 0 && c <= partition && !push(s, 0, c)) return false;
+  }
+  *n = at;
+  return true;
+}
+
 template <typename T, int BS, int G>
 hipError_t launch_g(const DecodeParams &P, int grid, hipStream_t st) {
   constexpr int NW = kWavesPerGroup;
@@ -1180,7 +1231,7 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
   for (int first = 0; first < n_items; ++first) {
     if (done[first]) continue;
     const int G = pick_group(items[first].num_q_heads / items[first].num_kv_heads);
-    DecodeParams P;
+    DecodeParams P = {};
     PlanParams PP;
     PP.partition = partition;
     int n_tables = 0;
@@ -1189,6 +1240,26 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
     P.partition = partition;
     P.last_block = static_cast<int32_t>(std::min<int64_t>(num_pool_blocks - 1, 0x7fffffff));
     P.n_items = 0;
+    P.n_host_pairs = 0;
+    // Host-enumerated units: every item of the launch group must come with its
+    // context lengths on the host, and the pairs must fit the kernel argument.
+    int pair_begin[MUXA_MAX_DECODE_ITEMS] = {0}, pair_end[MUXA_MAX_DECODE_ITEMS] = {0};
+    bool host_pairs = true;
+    {
+      int n_pairs = 0;
+      for (int i = first; i < n_items && host_pairs; ++i) {
+        const MuxDecodeItem &it = items[i];
+        if (done[i] || pick_group(it.num_q_heads / it.num_kv_heads) != G) continue;
+        if (it.num_seqs == 0 || it.max_context_len == 0) continue;
+        pair_begin[i] = n_pairs;
+        host_pairs = it.context_lens_host != nullptr &&
+                     enumerate_pairs_on_host(it.context_lens_host, it.num_seqs, it.max_context_len, partition,
+                                             P.pairs, &n_pairs);
+        pair_end[i] = n_pairs;
+      }
+      host_pairs = host_pairs && n_pairs > 0;
+      if (host_pairs) P.n_host_pairs = n_pairs;
+    }
     int64_t work = 0;
     for (int i = first; i < n_items; ++i) {
       if (done[i]) continue;
@@ -1209,6 +1280,21 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
       d.ws_ml = split ? reinterpret_cast<float *>(ws + plan[i].ml_off) : nullptr;
       d.counters = split ? reinterpret_cast<int32_t *>(ws + plan[i].counters_off) : nullptr;
       d.unit_table = nullptr;
+      d.pair_begin = pair_begin[i];
+      if (host_pairs) {
+        // The grid holds exactly this item's pairs; no table, no padding.
+        d.B = it.num_seqs;
+        d.Hq = it.num_q_heads;
+        d.Hkv = it.num_kv_heads;
+        d.ratio = it.num_q_heads / it.num_kv_heads;
+        d.max_blocks = it.max_blocks;
+        d.max_splits = plan[i].max_splits;
+        d.max_ctx = it.max_context_len;
+        d.work_begin = static_cast<int32_t>(work);
+        d.scale_log2 = it.scale * 1.4426950408889634f;
+        work += static_cast<int64_t>(pair_end[i] - pair_begin[i]) * (it.num_q_heads / G);
+        continue;
+      }
       if (plan[i].table_off != 0) {
         if (plan[i].units > 0x7fffffff) return MUXA_EUNSUPPORTED;
         PlanItem &t = PP.it[n_tables++];

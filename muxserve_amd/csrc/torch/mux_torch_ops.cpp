@@ -140,6 +140,7 @@ MuxDecodeItem decode_item(const at::Tensor &out, const at::Tensor &q, const at::
   it.max_blocks = static_cast<int32_t>(block_tables.size(3));
   it.max_context_len = static_cast<int32_t>(max_context_len);
   it.scale = static_cast<float>(scale);
+  it.context_lens_host = nullptr;
   return it;
 }
 

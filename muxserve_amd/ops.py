@@ -98,6 +98,10 @@ class DecodeCall:
     scale: float
     layer: int = 0
     total_context_len: int = 0    # host-side bound on sum(context_lens); 0 = unknown
+    # Optional host copy of context_lens (CPU int32 tensor [B], equal to the device
+    # tensor): small batches are then enumerated on the host and the launch does
+    # not read the device tensor.  Leave None under HIP graph capture.
+    context_lens_host: Optional[torch.Tensor] = None
 
     def to_item(self) -> _lib.MuxDecodeItem:
         bt, cl = self.block_tables, self.context_lens
@@ -122,6 +126,11 @@ class DecodeCall:
         it.max_blocks, it.max_context_len = max_blocks, int(self.max_context_len)
         it.scale = float(self.scale)
         it.total_context_len = int(self.total_context_len)
+        ch = self.context_lens_host
+        if ch is not None:
+            if ch.is_cuda or ch.dtype != torch.int32 or ch.dim() != 1 or ch.shape[0] != B or not ch.is_contiguous():
+                raise ValueError("context_lens_host: expected a contiguous CPU int32 [B] tensor")
+            it.context_lens_host = ch.data_ptr()      # self keeps the tensor alive over the call
         return it
 
 
@@ -192,9 +201,9 @@ def multi_decode_noalloc(calls: List[DecodeCall], k_pool: torch.Tensor, v_pool: 
 
 def paged_decode(out, q, k_pool, v_pool, block_tables, context_lens, max_context_len, scale,
                  layer: int = 0, partition_size: int = 0, workspace=None, stream=None,
-                 total_context_len: int = 0) -> None:
+                 total_context_len: int = 0, context_lens_host: Optional[torch.Tensor] = None) -> None:
     multi_decode([DecodeCall(out, q, block_tables, context_lens, max_context_len, scale, layer,
-                             total_context_len)],
+                             total_context_len, context_lens_host)],
                  k_pool, v_pool, partition_size, workspace, stream)
 
 

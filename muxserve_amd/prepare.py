@@ -78,6 +78,7 @@ def prepare_inputs(batch_scheduler: BatchScheduler, cache_alloc: Callable[[np.nd
     batch_reqs = batch_scheduler.get_batch_reqs()
     total_context_len = int(context_lens.sum()) if num_contexts else 0
 
+    context_lens_host = context_lens if num_contexts else None      # stays as written; the copy below only reads it
     slot_mapping = slot_mapping.to(device, non_blocking=True)
     block_tables = block_tables.to(device, non_blocking=True)
     input_tensor = input_tensor.to(device, non_blocking=True).long()            # llm_runtime.py:324-325
@@ -88,7 +89,7 @@ def prepare_inputs(batch_scheduler: BatchScheduler, cache_alloc: Callable[[np.nd
 
     input_metadata = InputMetadata(prompt_lens=prompt_lens, slot_mapping=slot_mapping, context_lens=context_lens,
                                    max_context_len=max_context_len, block_tables=block_tables,
-                                   total_context_len=total_context_len)
+                                   total_context_len=total_context_len, context_lens_host=context_lens_host)
     return input_tensor, input_positions, input_metadata, batch_reqs, preempted_reqs
 
 
@@ -113,6 +114,8 @@ def _prepare_on_device(sched, dt, batch_block_request, block_info, num_tokens, n
     desc_host = host[o_desc:o_info].view(n_entries, D)
     max_new = int(desc_host[:, 3].max()) if n_entries else 0
     total_context_len = int(host[o_ctx:o_ctx + num_contexts].sum()) if num_contexts else 0
+    # (the staging buffer is reused by the next step: the host copy is its own tensor)
+    context_lens_host = host[o_ctx:o_ctx + num_contexts].clone() if num_contexts else None
     preempted_reqs = sched.get_preempt_requests()
     batch_reqs = sched.get_batch_reqs()
 
@@ -125,5 +128,5 @@ def _prepare_on_device(sched, dt, batch_block_request, block_info, num_tokens, n
                                           max_num_blocks_per_seq if decoding else 0)
     input_metadata = InputMetadata(prompt_lens=prompt_lens, slot_mapping=slot_mapping, context_lens=context_lens,
                                    max_context_len=max_context_len, block_tables=block_tables,
-                                   total_context_len=total_context_len)
+                                   total_context_len=total_context_len, context_lens_host=context_lens_host)
     return input_tensor, input_positions, input_metadata, batch_reqs, preempted_reqs

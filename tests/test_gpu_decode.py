@@ -27,7 +27,7 @@ def _nan_pool(n, bs, dtype):
 
 
 def _decode_case(seed, ctx_lens, Hq, Hkv, bs, dtype=torch.float16, partition=0, num_layers=1, layer=0,
-                 q_in_qkv=False, extra_blocks=7, hint=False, repeat=1):
+                 q_in_qkv=False, extra_blocks=7, hint=False, repeat=1, host_lens=False):
     """Builds pool + tables on the host with the oracle's cache write, runs the
     GPU decode, returns (gpu_out fp32, oracle_out fp32)."""
     rng = np.random.Generator(np.random.PCG64(seed))
@@ -66,7 +66,8 @@ def _decode_case(seed, ctx_lens, Hq, Hkv, bs, dtype=torch.float16, partition=0, 
     for _ in range(repeat):     # repeated launches reuse the workspace (arrival counters must self-reset)
         out.fill_(7.0)
         ops.paged_decode(out, dq, dkp, dvp, dbt, dctx, int(ctx.max()), scale, layer=layer,
-                         partition_size=partition, total_context_len=int(ctx.sum()) if hint else 0)
+                         partition_size=partition, total_context_len=int(ctx.sum()) if hint else 0,
+                         context_lens_host=torch.from_numpy(ctx) if host_lens else None)
     torch.cuda.synchronize()
     got = out.float().cpu()
     assert (got[B:] == 7.0).all(), "padding rows of out must not be written"
@@ -246,6 +247,34 @@ def test_decode_split_context_equals_single_pass(partition):
     _check(got, want)
 
 
+@pytest.mark.parametrize("Hq,Hkv,dtype,partition", [(3, 3, torch.float16, 0), (4, 2, torch.bfloat16, 64),
+                                                     (8, 1, torch.float16, 128), (5, 5, torch.bfloat16, 512)])
+def test_decode_units_enumerated_on_the_host_equal_units_enumerated_on_the_device(Hq, Hkv, dtype, partition):
+    """With a host copy of the context lengths the (sequence, partition) pairs
+    travel in the kernel argument; the result must be the one the device-side
+    enumeration gives, bit for bit, and match the oracle.  Contexts cover no
+    tokens at all, one token, tile and partition boundaries, exact multiples
+    (no remainder unit) and long splits."""
+    _announce(f"decode host-enumerated units Hq={Hq} Hkv={Hkv} {dtype} partition={partition}")
+    ctx = [1, 0, 64, 65, 200, 256, 257, 512, 513, 777, 0, 1024, 1500, 16]
+    dev_got, want = _decode_case(11, ctx, Hq, Hkv, 16, dtype=dtype, partition=partition, repeat=2)
+    host_got, _ = _decode_case(11, ctx, Hq, Hkv, 16, dtype=dtype, partition=partition, repeat=2, host_lens=True)
+    live = torch.tensor(ctx) > 0
+    assert torch.equal(host_got[live], dev_got[live])
+    _check(host_got[live], want[live], out_dtype=dtype)
+    assert (host_got[~live] == 7.0).all(), "sequences without tokens must not be written"
+
+
+def test_decode_host_lens_too_many_pairs_falls_back_to_the_device_enumeration():
+    """More pairs than the kernel argument holds (here 400 sequences): the call
+    silently takes the device-side path and still matches the oracle."""
+    _announce("decode host lens, 400 sequences")
+    rng = np.random.Generator(np.random.PCG64(5))
+    ctx = rng.integers(1, 200, size=400)
+    got, want = _decode_case(12, ctx, 2, 2, 16, partition=128, host_lens=True)
+    _check(got, want)
+
+
 @pytest.mark.parametrize("B", [65, 130, 300])
 @pytest.mark.parametrize("hint", [False, True])
 def test_decode_more_sequences_than_a_wave(B, hint):
@@ -347,6 +376,17 @@ def test_multi_decode_three_models_one_launch_matches_separate_launches():
         ops.paged_decode(m.out, m.q, dk, dv, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
                          partition_size=256)
     torch.cuda.synchronize()
+    # The same fused launch with the units enumerated on the host.
+    host_calls = [ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                                 context_lens_host=torch.from_numpy(np.ascontiguousarray(m.context_lens, dtype=np.int32)))
+                  for m in models]
+    separate = [m.out.clone() for m in models]
+    for m in models:
+        m.out.zero_()
+    ops.multi_decode(host_calls, dk, dv, partition_size=256)
+    torch.cuda.synchronize()
+    for m, sep in zip(models, separate):
+        assert torch.equal(m.out, sep), "host-enumerated and device-enumerated launches must agree bitwise"
     ks, vs, tables = workloads.compact_to_host(dk, dv, models, bs)
     for m, f, t in zip(models, fused, tables):
         assert torch.equal(f, m.out), "fused and separate launches must agree bitwise"
