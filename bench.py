@@ -332,7 +332,7 @@ def bench_gqa_long(args):
     # The yardstick: the same blocks read by the bare gather-read probe.
     used = [torch.from_numpy(m.used_blocks(bs).astype(np.int32)).to(dev) for m in sets]
     sink = torch.zeros((1,), dtype=torch.int32, device=dev)
-    probe_ms = _time(lambda i: ops.probe_gather_read(k_pool, v_pool, used[i % len(used)], sink), args.steps, args.warmup)
+    probe_ms = _time(lambda i: workloads.probe_gather_read(k_pool, v_pool, used[i % len(used)], sink), args.steps, args.warmup)
     probe_bytes = float(np.mean([u.numel() * 8192 for u in used]))
     cfg = {"workload": "gqa_long", "shape": "Hq64/Hkv8, B=64, ctx U[2048,8192], bf16", "pool_gb": round(N * 8192 / 1e9, 1),
            "bytes_per_step": int(nbytes), "partition": args.partition}
@@ -640,7 +640,7 @@ def main():
     # The yardstick: the same blocks read by the bare gather-read probe (the decode
     # kernel's loads, no table walk, no arithmetic), same rotation of the sets.
     sink = torch.zeros((1,), dtype=torch.int32, device=dev)
-    probe_ms = _time(lambda i: ops.probe_gather_read(k_pool, v_pool, sets[i % len(sets)][2], sink),
+    probe_ms = _time(lambda i: workloads.probe_gather_read(k_pool, v_pool, sets[i % len(sets)][2], sink),
                      args.steps, args.warmup)
     probe_bytes = sum(int(s[2].numel()) * 8192 * v for s, v in
                       zip(sets, [len(range(i, args.steps, len(sets))) for i in range(len(sets))])) / args.steps

@@ -304,18 +304,6 @@ int32_t mux_build_step_inputs(int32_t *mirror, int32_t max_rows, int32_t max_blo
                               int64_t *slot_mapping, int32_t *block_tables, int32_t max_blocks_out,
                               void *stream);
 
-/* ---- Measuring aid -------------------------------------------------------
- * No reference counterpart.  Reads the K and V head-blocks named by block_ids
- * (DEVICE int32 [n_blocks]; entries outside the pool are clamped) with the load
- * pattern of the decode kernel - four blocks per wave, all loads in flight - and
- * does nothing else: the rate it reaches is what the memory system gives to
- * whole 4 KiB blocks scattered over the pool, the yardstick next to the
- * attention kernel's own rate.  block_size must be 16.  sink: DEVICE uint32 [1]
- * (only ever written when the folded data equals an arbitrary constant). */
-int32_t mux_probe_gather_read(const void *k_pool, const void *v_pool, int64_t num_pool_blocks,
-                              const int32_t *block_ids, int64_t n_blocks, int32_t block_size,
-                              uint32_t *sink, void *stream);
-
 /* ---- CU-masked streams ---------------------------------------------------
  * Replacement for the reference's per-process MPS share
  * (CUDA_MPS_ACTIVE_THREAD_PERCENTAGE, muxserve/muxsched/launcher.py:54-61):

@@ -11,9 +11,11 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 # alternative build of the same ABI (e.g. one compiled with other flags).
 HOST_LIB_PATH = os.environ.get("MUXSERVE_HOST_LIB", os.path.join(_PKG, "libmuxhost.so"))
 ATTN_LIB_PATH = os.environ.get("MUXSERVE_ATTN_LIB", os.path.join(_PKG, "libmuxattn.so"))
+PROBE_LIB_PATH = os.environ.get("MUXSERVE_PROBE_LIB", os.path.join(_PKG, "libmuxprobe.so"))
 
 _host = None
 _attn = None
+_probe = None
 
 c_i32 = ctypes.c_int32
 c_i64 = ctypes.c_int64
@@ -143,7 +145,6 @@ ATTN_SIGNATURES = {
                                   c_vp, c_sz, c_vp]),
     "mux_build_step_inputs": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_i32, c_vp, c_i64, c_i32,
                                       c_i32, c_vp, c_vp, c_i32, c_vp]),
-    "mux_probe_gather_read": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp]),
     "mux_stream_create_cu_range": (c_i32, [c_vp, c_i32, c_i32, c_vp]),
     "mux_stream_destroy": (c_i32, [c_vp]),
     "mux_device_cu_info": (c_i32, [c_vp]),
@@ -162,6 +163,18 @@ def attn():
         fn.argtypes = args
     _attn = lib
     return lib
+
+
+def probe():
+    """libmuxprobe.so (muxserve_amd/csrc/probe/mux_probe.h): the bare gather-read
+    kernel bench.py times next to the attention kernel.  Not part of the product."""
+    global _probe
+    if _probe is None:
+        lib = _open(PROBE_LIB_PATH)
+        lib.mux_probe_gather_read.restype = c_i32
+        lib.mux_probe_gather_read.argtypes = [c_vp, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp]
+        _probe = lib
+    return _probe
 
 
 ATTN_ERRORS = {-1: "invalid argument", -2: "unsupported shape or dtype",

@@ -3,6 +3,7 @@
     libmuxhost.so  - g++,   pure host C++ (allocator + batch builder)
     libmuxattn.so  - hipcc, gfx950 kernels + their C ABI
     libmuxtorch.so - g++,   thin TORCH_LIBRARY operators over libmuxattn.so's C ABI
+    libmuxprobe.so - hipcc, a bare gather-read kernel: bench.py's yardstick, not product
 
 Run as ``python -m muxserve_amd.build``.  Nothing here runs at import time of
 the package: the loaders in muxserve_amd._lib only open what this step built
@@ -20,12 +21,14 @@ CSRC = os.path.join(PKG, "csrc")
 HOST_LIB = os.path.join(PKG, "libmuxhost.so")
 ATTN_LIB = os.path.join(PKG, "libmuxattn.so")
 TORCH_LIB = os.path.join(PKG, "libmuxtorch.so")
+PROBE_LIB = os.path.join(PKG, "libmuxprobe.so")
+PROBE_SOURCES = [os.path.join(CSRC, "probe", "probe.hip")]
 TORCH_SOURCES = [os.path.join(CSRC, "torch", "mux_torch_ops.cpp")]
 
 HOST_SOURCES = [os.path.join(CSRC, "host", f) for f in ("kv_storage.cpp", "batch_scheduler.cpp")]
 HIP_SOURCES = [os.path.join(CSRC, "hip", f) for f in (
     "cache_write.hip", "paged_decode.hip", "prefill.hip", "rotary.hip", "model_ops.hip", "sampler.hip",
-    "step_tables.hip", "probe.hip", "runtime.hip")]
+    "step_tables.hip", "runtime.hip")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # Packed-FP32 instruction selection is switched off for every device
@@ -53,6 +56,11 @@ def build_hip(extra=()):
     return ATTN_LIB
 
 
+def build_probe():
+    _run([HIPCC, *HIP_FLAGS, f"-I{os.path.join(CSRC, 'probe')}", *PROBE_SOURCES, "-o", PROBE_LIB])
+    return PROBE_LIB
+
+
 def build_torch():
     """The operator library: host C++ only (no device code), linked against
     torch's libraries and libmuxattn.so next to it."""
@@ -73,8 +81,9 @@ def build_all():
     build_host()
     build_hip()
     build_torch()
+    build_probe()
 
 
 if __name__ == "__main__":
     what = sys.argv[1] if len(sys.argv) > 1 else "all"
-    {"host": build_host, "hip": build_hip, "torch": build_torch, "all": build_all}[what]()
+    {"host": build_host, "hip": build_hip, "torch": build_torch, "probe": build_probe, "all": build_all}[what]()

@@ -10,7 +10,10 @@
 // four V blocks as consecutive 1 KiB runs; all 32 loads are non-temporal and in
 // flight together.  The data is folded into one word that is never stored
 // unless it equals an arbitrary constant, so the loads cannot be optimised away.
-#include "mux_common.h"
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mux_probe.h"
 
 namespace mux {
 
@@ -50,16 +53,15 @@ extern "C" int32_t mux_probe_gather_read(const void *k_pool, const void *v_pool,
                                          const int32_t *block_ids, int64_t n_blocks, int32_t block_size,
                                          uint32_t *sink, void *stream) {
   using namespace mux;
-  if (!k_pool || !v_pool || !sink || num_pool_blocks <= 0 || n_blocks < 0) return MUXA_EINVAL;
-  if (n_blocks > 0 && !block_ids) return MUXA_EINVAL;
-  if ((reinterpret_cast<uintptr_t>(k_pool) | reinterpret_cast<uintptr_t>(v_pool)) & 15u) return MUXA_EINVAL;
-  if (block_size != 16) return MUXA_EUNSUPPORTED;       // 4 KiB head-blocks: 256 chunks of 16 bytes
-  if (n_blocks == 0) return MUXA_OK;
+  if (!k_pool || !v_pool || !sink || num_pool_blocks <= 0 || n_blocks < 0) return -1;
+  if (n_blocks > 0 && !block_ids) return -1;
+  if ((reinterpret_cast<uintptr_t>(k_pool) | reinterpret_cast<uintptr_t>(v_pool)) & 15u) return -1;
+  if (block_size != 16) return -2;       // 4 KiB head-blocks: 256 chunks of 16 bytes
+  if (n_blocks == 0) return 0;
   const int64_t n_wg = (n_blocks + 15) / 16;
-  if (n_wg > 0x7fffffff) return MUXA_EUNSUPPORTED;
+  if (n_wg > 0x7fffffff) return -2;
   hipLaunchKernelGGL(probe_gather_read_kernel, dim3(static_cast<uint32_t>(n_wg)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), static_cast<const uint4 *>(k_pool),
                      static_cast<const uint4 *>(v_pool), block_ids, n_blocks, num_pool_blocks, sink);
-  MUX_HIP_TRY(hipGetLastError());
-  return MUXA_OK;
+  return hipGetLastError() == hipSuccess ? 0 : -4;
 }

@@ -381,23 +381,6 @@ def greedy_sample(embedding: torch.Tensor, hidden_states: torch.Tensor, vocab_si
     return out[:num_rows]
 
 
-def probe_gather_read(k_pool: torch.Tensor, v_pool: torch.Tensor, block_ids: torch.Tensor,
-                      sink: Optional[torch.Tensor] = None, stream=None) -> None:
-    """Measuring aid: reads the K and V head-blocks named by block_ids (int32,
-    device) with the decode kernel's load pattern and nothing else.  Bytes read:
-    block_ids.numel() * 8192 at block size 16."""
-    _need_cuda(k_pool, v_pool, block_ids)
-    bs = _check_pools(k_pool, v_pool)
-    if block_ids.dtype != torch.int32 or block_ids.dim() != 1 or not block_ids.is_contiguous():
-        raise ValueError("block_ids: expected contiguous int32 [n]")
-    if sink is None:
-        sink = torch.zeros((1,), dtype=torch.int32, device=k_pool.device)
-    rc = _lib.attn().mux_probe_gather_read(k_pool.data_ptr(), v_pool.data_ptr(), k_pool.shape[0],
-                                           block_ids.data_ptr(), block_ids.numel(), bs, sink.data_ptr(),
-                                           _stream_ptr(stream))
-    _lib.check_attn(rc, "mux_probe_gather_read")
-
-
 class CUMaskedStream:
     """A HIP stream restricted to a share of the GPU's compute units (the
     replacement for a per-process MPS percentage).  Usable wherever a stream is

@@ -241,3 +241,22 @@ def prefill_flops(prompt_lens, num_q_heads, head_size=HEAD_SIZE):
     """QK^T and PV over the causal triangle: 4 * Hq * D * sum L (L + 1) / 2."""
     lens = np.asarray(prompt_lens, dtype=np.float64)
     return 4.0 * num_q_heads * head_size * float((lens * (lens + 1) / 2).sum())
+
+
+def probe_gather_read(k_pool: torch.Tensor, v_pool: torch.Tensor, block_ids: torch.Tensor,
+                      sink: Optional[torch.Tensor] = None, stream=None) -> None:
+    """Measuring aid (libmuxprobe.so, not the product library): reads the K and V
+    head-blocks named by block_ids (int32, device) with the decode kernel's load
+    pattern and nothing else.  Bytes read: block_ids.numel() * 8192 at block
+    size 16."""
+    from . import _lib, ops
+    ops._need_cuda(k_pool, v_pool, block_ids)
+    bs = ops._check_pools(k_pool, v_pool)
+    if block_ids.dtype != torch.int32 or block_ids.dim() != 1 or not block_ids.is_contiguous():
+        raise ValueError("block_ids: expected contiguous int32 [n]")
+    if sink is None:
+        sink = torch.zeros((1,), dtype=torch.int32, device=k_pool.device)
+    rc = _lib.probe().mux_probe_gather_read(k_pool.data_ptr(), v_pool.data_ptr(), k_pool.shape[0],
+                                            block_ids.data_ptr(), block_ids.numel(), bs, sink.data_ptr(),
+                                            ops._stream_ptr(stream))
+    _lib.check_attn(rc, "mux_probe_gather_read")

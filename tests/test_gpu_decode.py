@@ -232,6 +232,35 @@ def test_decode_config1_shape():
     _check(got, want)
 
 
+def test_decode_config1_with_its_own_tables():
+    """The same configuration with the tables the workload itself defines: one
+    seeded permutation of a 4096-group pool (4096 * 32 head-blocks), a token
+    block's 32 heads at ids group * 32 + head.  Checked against the oracle
+    reading the same pool through the same tables."""
+    _announce("decode config 1, own tables")
+    bs = 16
+    models, N = workloads.config1(seed=0)
+    m = models[0]
+    assert N == 4096 * 32 and m.block_tables.shape[:3] == (1, 8, 32)
+    groups = m.block_tables[0, :, 0, :] // 32
+    for s, c in enumerate(m.context_lens):
+        n = (int(c) + bs - 1) // bs
+        assert (m.block_tables[0, s, :, :n] == groups[s, :n][None, :] * 32 + np.arange(32)[:, None]).all()
+    dk, dv = allocate_gpu_cache(N, bs, DEV)
+    dk.fill_(float("nan"))
+    dv.fill_(float("nan"))
+    workloads.fill_blocks(dk, dv, m.used_blocks(bs), seed=1)
+    m.to_device(DEV, torch.float16, seed=2)
+    for host_lens in (None, torch.from_numpy(np.ascontiguousarray(m.context_lens, dtype=np.int32))):
+        m.out.fill_(7.0)
+        ops.paged_decode(m.out, m.q, dk, dv, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                         context_lens_host=host_lens)
+        torch.cuda.synchronize()
+        want = orc.paged_decode(m.q.cpu(), dk.cpu(), dv.cpu(), torch.from_numpy(m.block_tables), m.context_lens,
+                                m.scale)
+        _check(m.out[:m.batch].float().cpu(), want)
+
+
 @pytest.mark.parametrize("ctx", [[1], [2, 15, 16, 17], [63, 64, 65, 127, 128, 129], [255, 256, 257, 300]])
 def test_decode_boundaries(ctx):
     _announce(f"decode boundaries ctx={ctx}")
@@ -446,7 +475,7 @@ def test_decode_rejects_bad_arguments():
     torch.cuda.synchronize()
 
 
-def test_decode_config2_full_size_pool():
+def test_decode_config2_full_size_pool(full_size_pool_memory):
     """Headline workload at its real size: pool = 60% of HBM, three models,
     ids scattered over the whole pool.  Checked against the oracle on a compact
     host copy of the referenced blocks (attention is invariant under relabelling
@@ -455,7 +484,7 @@ def test_decode_config2_full_size_pool():
     bs = 16
     total = torch.cuda.get_device_properties(0).total_memory
     N = num_gpu_blocks(0.6, total, bs)
-    dk, dv = allocate_gpu_cache(N, bs, DEV)
+    dk, dv = full_size_pool_memory(N, bs, torch.float16)
     models, need = workloads.config2(seed=0, num_pool_blocks=N)
     used = np.concatenate([m.used_blocks(bs) for m in models])
     assert used.max() > N // 2, "ids must span the pool"
@@ -529,15 +558,15 @@ def test_gather_read_probe_runs_and_rejects_what_it_cannot_read():
     sink = torch.zeros((1,), dtype=torch.int32, device=DEV)
     for n in (1, 3, 4, 17, 1000):
         ids = torch.randint(-5, N + 5, (n,), dtype=torch.int32, device=DEV)
-        ops.probe_gather_read(k_pool, v_pool, ids, sink)
-    ops.probe_gather_read(k_pool, v_pool, torch.zeros((0,), dtype=torch.int32, device=DEV), sink)
+        workloads.probe_gather_read(k_pool, v_pool, ids, sink)
+    workloads.probe_gather_read(k_pool, v_pool, torch.zeros((0,), dtype=torch.int32, device=DEV), sink)
     torch.cuda.synchronize()
     assert torch.equal(k_pool, k0) and torch.equal(v_pool, v0)
     k8, v8 = allocate_gpu_cache(64, 8, DEV)
     with pytest.raises(RuntimeError):
-        ops.probe_gather_read(k8, v8, torch.zeros((4,), dtype=torch.int32, device=DEV), sink)
-    assert _lib.attn().mux_probe_gather_read(None, v_pool.data_ptr(), N, sink.data_ptr(), 4, 16, sink.data_ptr(),
-                                             None) == -1      # MUXA_EINVAL
+        workloads.probe_gather_read(k8, v8, torch.zeros((4,), dtype=torch.int32, device=DEV), sink)
+    assert _lib.probe().mux_probe_gather_read(None, v_pool.data_ptr(), N, sink.data_ptr(), 4, 16, sink.data_ptr(),
+                                             None) == -1      # invalid argument
 
 
 @pytest.mark.parametrize("seed", range(24))

@@ -1,12 +1,14 @@
 """prepare_inputs with the device-side builder (DeviceBlockTables) against
-prepare_inputs on the reference-shaped host path: the same scenario is driven
-through two scheduler/allocator pairs in lockstep and every tensor the model
+prepare_inputs on the reference-shaped host path and against the oracle's
+restatement of the reference's prepare_inputs: the same scenario is driven
+through three scheduler/allocator pairs in lockstep and every tensor the model
 code receives must be bit-identical (block-table entries the reference leaves
 undefined excepted)."""
 import numpy as np
 import pytest
 import torch
 
+from oracle import host_oracle
 from muxserve_amd.batch_scheduler import BatchScheduler
 from muxserve_amd.device_tables import DeviceBlockTables
 from muxserve_amd.memory_manager import KVStorage
@@ -20,13 +22,45 @@ def _pair(L, H, bs, N, rows, max_seq_len=1024):
     a = (KVStorage(N), BatchScheduler(L, H, max_seq_len, bs))
     b = (KVStorage(N), BatchScheduler(L, H, max_seq_len, bs))
     dt = DeviceBlockTables(b[1], rows, DEV)
+    _ORACLE[id(dt)] = (host_oracle.KVStorage(N), host_oracle.BatchScheduler(L, H, max_seq_len, bs))
     return a, b, dt
+
+
+_ORACLE = {}       # the oracle's allocator and batch builder that shadow a pair
+
+
+def _oracle_do(dt, fn):
+    st, sc = _ORACLE[id(dt)]
+    fn(st, sc)
+
+
+def _against_oracle(ref, got, bs):
+    """The device-built step against the oracle's reference-shaped tensors."""
+    tok, pos, md, batch_reqs, preempted = got
+    T = sum(ref["prompt_lens"]) + int(ref["context_lens"].numel())
+    assert tok.dtype == torch.int64 and tok.shape == ref["input_tensor"].shape
+    assert torch.equal(tok.cpu()[:T], ref["input_tensor"][:T]) and torch.equal(pos.cpu()[:T], ref["input_positions"][:T])
+    assert md.slot_mapping.dtype == torch.int64 and torch.equal(md.slot_mapping.cpu(), ref["slot_mapping"])
+    assert md.context_lens.dtype == torch.int32 and torch.equal(md.context_lens.cpu(), ref["context_lens"])
+    assert md.max_context_len == ref["max_context_len"] and md.prompt_lens == [int(x) for x in ref["prompt_lens"]]
+    assert [list(x) for x in batch_reqs] == [list(x) for x in ref["batch_reqs"]]
+    assert list(preempted) == list(ref["preempted_reqs"])
+    if ref["max_context_len"] > 0:
+        rt, gt = ref["block_tables"], md.block_tables.cpu()
+        assert gt.shape == rt.shape and gt.dtype == torch.int32
+        for c, n in enumerate(ref["context_lens"].tolist()):
+            valid = (n + bs - 1) // bs
+            assert torch.equal(gt[:, c, :, :valid], rt[:, c, :, :valid]), f"sequence {c}"
+    else:
+        assert md.block_tables.numel() == 0 and ref["block_tables"].numel() == 0
 
 
 def _both(a, b, dt, L, H, ids, last, bs):
     ra = prepare_inputs(a[1], lambda r: a[0].allocate_batch(r, L, H), ids, last, DEV, permuted_tables=False)
     rb = prepare_inputs(b[1], lambda r: b[0].allocate_batch(r, L, H), ids, last, DEV, device_tables=dt)
     torch.cuda.synchronize()
+    ost, osc = _ORACLE[id(dt)]
+    _against_oracle(host_oracle.prepare_inputs(osc, ost, L, H, ids, last), rb, bs)
     (ta, pa, ma, qa, ea), (tb, pb, mb, qb, eb) = ra, rb
     assert torch.equal(ta, tb) and torch.equal(pa, pb) and qa == qb and ea == eb
     assert ma.prompt_lens == mb.prompt_lens and ma.max_context_len == mb.max_context_len
@@ -55,19 +89,21 @@ def test_device_built_step_inputs_equal_the_host_built_ones(L, H, bs):
         prompt = rng.integers(0, 32000, size=p).astype(np.int32)
         a[1].add_request(prompt, i, 64)
         b[1].add_request(prompt, i, 64)
+        _oracle_do(dt, lambda st, sc: sc.add_request(prompt, i, 64))
     ids = list(range(len(lens)))
     _both(a, b, dt, L, H, ids[:5], [], bs)                         # two prefill steps
     _both(a, b, dt, L, H, ids[5:], [], bs)
     for step in range(bs + 3):                                      # decode across block boundaries
         order = ids[::-1] if step % 2 else ids
         _both(a, b, dt, L, H, order, [step + 1] * len(ids), bs)
-    for st, sc in (a, b):                                           # release, then new requests reuse rows
+    for st, sc in (a, b, _ORACLE[id(dt)]):                          # release, then new requests reuse rows
         st.free_batch([0, 4, 8])
         sc.release_requests([0, 4, 8])
     for rid, p in ((20, 33), (21, 1), (22, 3 * bs)):
         prompt = rng.integers(0, 32000, size=p).astype(np.int32)
         a[1].add_request(prompt, rid, 64)
         b[1].add_request(prompt, rid, 64)
+        _oracle_do(dt, lambda st, sc: sc.add_request(prompt, rid, 64))
     _both(a, b, dt, L, H, [20, 21, 22], [], bs)
     live = [1, 2, 3, 5, 6, 7, 20, 21, 22]
     for step in range(4):
@@ -83,6 +119,7 @@ def test_device_built_step_inputs_with_preemption():
         prompt = np.arange(p, dtype=np.int32)
         a[1].add_request(prompt, i, 32)
         b[1].add_request(prompt, i, 32)
+        _oracle_do(dt, lambda st, sc: sc.add_request(prompt, i, 32))
     cut = _both(a, b, dt, L, H, [0, 1, 2, 3], [], bs)
     assert cut, "the pool was meant to be too small for the batch"
     alive = [r for r in [0, 1, 2, 3] if r not in cut]

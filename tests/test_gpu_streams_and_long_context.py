@@ -56,13 +56,83 @@ def test_cu_masked_streams_run_prefill_and_decode_concurrently_and_correctly():
         ops.CUMaskedStream(50, 50)
 
 
-def test_long_context_gqa_bf16_full_size_pool():
+def test_colocated_prefill_and_decode_at_the_benchmark_shapes():
+    """The colocated configuration at its real shapes: a 30B-shaped prefill (52
+    heads x 128, 4 prompts x 1024 tokens, fp16) on 40% of the compute units
+    while a 7B-shaped decode (32 heads, batch 64, contexts uniform [512, 1024],
+    block size 16) runs on the other 60%, both streams kept busy for several
+    rounds, cache write of the prefill included (bit-exact).  The oracle runs
+    on a subset: 4 heads of two prompts, and 6 sequences of the decode batch."""
+    print("[case] colocated prefill + decode, benchmark shapes", flush=True)
+    bs, N = 16, 160000
+    Hp, Hd = 52, 32
+    rng = np.random.Generator(np.random.PCG64(44))
+    g = torch.Generator().manual_seed(44)
+    k_pool, v_pool = allocate_gpu_cache(N, bs, DEV)
+    ctx = rng.integers(512, 1025, size=64).astype(np.int32)
+    need_d = int(((ctx + bs - 1) // bs).sum()) * Hd
+    lens = [1024] * 4
+    T = sum(lens)
+    need_p = (T // bs) * Hp
+    ids = rng.choice(N, size=need_d + need_p, replace=False)
+    bt, _ = workloads.build_tables(ctx, Hd, bs, ids[:need_d])
+    dec = workloads.DecodeModel("7b", Hd, Hd, ctx, bt)
+    workloads.fill_blocks(k_pool, v_pool, dec.used_blocks(bs), seed=45)
+    dec.to_device(DEV, torch.float16, seed=46)
+    slots, _ = workloads.prefill_slot_mapping(lens, Hp, bs, ids[need_d:])       # int64 [T, 1, Hp]
+    qkv = torch.randn((T, 3 * Hp * D), generator=g).half()
+    dqkv = qkv.to(DEV)
+    q, k, v = dqkv.split([Hp * D] * 3, dim=-1)
+    dslots = torch.from_numpy(slots).to(DEV)
+    cu = torch.tensor([0, 1024, 2048, 3072, 4096], dtype=torch.int32, device=DEV)
+    pout = torch.zeros((T, Hp * D), dtype=torch.float16, device=DEV)
+    s_prefill, s_decode = ops.CUMaskedStream(0, 40), ops.CUMaskedStream(40, 100)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        with torch.cuda.stream(s_prefill.torch_stream):
+            ops.prefill_causal(pout, q, k, v, cu, 1024, D ** -0.5, Hp)
+            ops.reshape_and_cache(k, v, k_pool, v_pool, dslots)
+        with torch.cuda.stream(s_decode.torch_stream):
+            for _ in range(4):          # a decode step is several times shorter than the prefill
+                ops.paged_decode(dec.out, dec.q, k_pool, v_pool, dec.d_block_tables, dec.d_context_lens,
+                                 dec.max_context_len, dec.scale, total_context_len=int(ctx.sum()),
+                                 context_lens_host=torch.from_numpy(ctx))
+    s_prefill.synchronize()
+    s_decode.synchronize()
+    # prefill: heads 0, 17, 30, 51 of prompts 1 and 3 (causal attention is per head and per prompt)
+    heads = [0, 17, 30, 51]
+    cols = torch.cat([torch.arange(h * D, (h + 1) * D) for h in heads])
+    qh, kh, vh = (qkv[:, o * Hp * D:(o + 1) * Hp * D] for o in range(3))
+    for p in (1, 3):
+        rows = slice(1024 * p, 1024 * (p + 1))
+        want = orc.prefill_causal(qh[rows][:, cols], kh[rows][:, cols], vh[rows][:, cols], [1024], D ** -0.5,
+                                  len(heads))
+        got = pout[rows].float().cpu()[:, cols]
+        assert (got - want).abs().max().item() <= 2e-3
+    # the prefill's cache write, bit-exact on every slot it names
+    hk, hv = orc.allocate_pool(N, bs, torch.float16)
+    orc.reshape_and_cache(kh, vh, hk, hv, torch.from_numpy(slots))
+    pblocks = torch.from_numpy(np.unique(slots // bs))
+    assert torch.equal(k_pool.cpu()[pblocks].view(torch.int16), hk[pblocks].view(torch.int16))
+    assert torch.equal(v_pool.cpu()[pblocks].view(torch.int16), hv[pblocks].view(torch.int16))
+    # decode: six sequences (shortest, longest, four more), all heads
+    pick = sorted({int(np.argmin(ctx)), int(np.argmax(ctx)), 0, 21, 42, 63})
+    sub = workloads.DecodeModel("7b", Hd, Hd, ctx[pick].copy(), dec.block_tables[:, pick].copy(), dec.scale)
+    ks, vs, tables = workloads.compact_to_host(k_pool, v_pool, [sub], bs)
+    want_d = orc.paged_decode(dec.q[pick].cpu(), ks, vs, tables[0], sub.context_lens, dec.scale)
+    assert (dec.out[pick].float().cpu() - want_d).abs().max().item() <= 2e-3
+    assert torch.isfinite(dec.out[:64].float()).all() and torch.isfinite(pout.float()).all()
+    s_prefill.close()
+    s_decode.close()
+
+
+def test_long_context_gqa_bf16_full_size_pool(full_size_pool_memory):
     """Config 5 at its real shape.  The oracle runs on a compact host copy of
     the referenced blocks for a subset of the sequences."""
     print("[case] long-context gqa", flush=True)
     bs = 16
     N = int(200e9) // 8192 // 128 * 128
-    k_pool, v_pool = allocate_gpu_cache(N, bs, DEV, dtype=torch.bfloat16)
+    k_pool, v_pool = full_size_pool_memory(N, bs, torch.bfloat16)
     models, need = workloads.config5(seed=0, num_pool_blocks=N)
     m = models[0]
     used = m.used_blocks(bs)
