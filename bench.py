@@ -206,6 +206,32 @@ def bench_cache_write(args):
     ms_d = _time(lambda _: [ops.reshape_and_cache(k, v, k_pool, v_pool, s) for k, v, s, b, hk in dec],
                  args.steps, args.warmup)
     bytes_d = sum(workloads.cache_write_bytes(b, hk) for *_, b, hk in dec)
+    # the same three writes in one launch; with the rotary embedding fused; and the whole
+    # attention part of a three-model decode step: rope + cache write (one launch) + paged
+    # decode attention (one launch) over the mix's contexts
+    plain_calls = [ops.CacheWriteCall(k, v, s) for k, v, s, b, hk in dec]
+    plain_items = ops.cache_write_items(plain_calls, k_pool.dtype)      # checked once, not per launch
+    ms_d1 = _time(lambda _: ops.multi_reshape_and_cache(plain_items, k_pool, v_pool), args.steps, args.warmup)
+    from muxserve_amd.attention import build_cos_sin_cache
+    cos_sin = build_cos_sin_cache(D, 4096, 10000.0, dev)
+    mix, _need = workloads.config2(seed=args.seed + 1, num_pool_blocks=N)
+    rope_calls, dcalls = [], []
+    for m, (k, v, s, b, hk) in zip(mix, dec):
+        m.to_device(dev, torch.float16, seed=7)
+        pos = torch.from_numpy(m.context_lens.astype(np.int64) - 1).to(dev)
+        rope_calls.append(ops.CacheWriteCall(k, v, s, positions=pos, cos_sin=cos_sin, q=m.q[:b]))
+        dcalls.append(ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                                     total_context_len=int(m.context_lens.sum()),
+                                     context_lens_host=torch.from_numpy(np.ascontiguousarray(m.context_lens,
+                                                                                             dtype=np.int32))))
+    rope_items = ops.cache_write_items(rope_calls, k_pool.dtype)
+    ms_dr = _time(lambda _: ops.multi_reshape_and_cache(rope_items, k_pool, v_pool), args.steps, args.warmup)
+
+    def attention_part(_):
+        ops.multi_reshape_and_cache(rope_items, k_pool, v_pool)
+        ops.multi_decode(dcalls, k_pool, v_pool)
+
+    ms_step = _time(attention_part, args.steps, args.warmup)
     # prefill-shaped
     # Five sources and five disjoint sets of pool blocks in rotation (1.1 GB), so
     # that neither k/v nor the pool lines come from the 256 MB last-level cache.
@@ -230,7 +256,9 @@ def bench_cache_write(args):
     cfg = {"workload": "cache_write", "prefill_shape": "52 heads x 4096 tokens", "prefill_bytes": bytes_p,
            "same_buffers_every_step_ms": ms_warm, "same_buffers_every_step_gbs": bytes_p / (ms_warm * 1e-3) / 1e9,
            "decode_shape": "7b/13b/30b, 56 tokens, three launches", "decode_ms": ms_d, "decode_bytes": bytes_d,
-           "decode_gbs": bytes_d / (ms_d * 1e-3) / 1e9}
+           "decode_gbs": bytes_d / (ms_d * 1e-3) / 1e9,
+           "decode_one_fused_launch_ms": ms_d1, "decode_one_fused_launch_with_rope_ms": ms_dr,
+           "decode_step_rope_write_attention_two_launches_ms": ms_step}
     roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
             "traffic": bytes_p * CACHE_WRITE_TRAFFIC_RATIO,
             "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiles/other_kernels_kernel_trace.txt",

@@ -238,6 +238,38 @@ int32_t mux_rope_reshape_and_cache(const int64_t *positions, void *q, int64_t q_
                                    int32_t num_kv_heads, int32_t head_size, int32_t block_size,
                                    int32_t dtype, void *stream);
 
+/* The cache writes of one step of up to MUXA_MAX_DECODE_ITEMS colocated models
+ * in ONE launch (the write-side counterpart of mux_multi_decode): the reference
+ * issues one reshape_and_cache per model and layer (models/llama.py:159-161);
+ * models that share the pool, block size and dtype and run the same step can
+ * share the grid, which removes the per-launch latency that dominates a decode
+ * step's write of a few dozen tokens.  Field meanings are those of
+ * mux_rope_reshape_and_cache / mux_reshape_and_cache; either every item rotates
+ * (positions != NULL: q and k rotated in place, rotated k scattered) or none
+ * does (positions == NULL: plain scatter; q, cos_sin, rotary fields unused).
+ * Result: bit-identical to the per-model calls.  `items` is a HOST array. */
+typedef struct MuxCacheWriteItem {
+  const int64_t *positions;      /* [num_tokens] or NULL (no rotation) */
+  void *q;                       /* rotated in place; may be NULL */
+  int64_t q_row_stride;
+  void *k;                       /* rotated in place when positions != NULL */
+  const void *v;
+  int64_t kv_row_stride;
+  const float *cos_sin;          /* [max_position, rotary_dim] = [cos | sin] */
+  const int64_t *slot_mapping;   /* base of the int64 [num_tokens, L, Hkv] tensor */
+  int32_t max_position;
+  int32_t rotary_dim;
+  int32_t layer;
+  int32_t num_layers;
+  int32_t num_tokens;
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+} MuxCacheWriteItem;
+
+int32_t mux_multi_rope_reshape_and_cache(const MuxCacheWriteItem *items, int32_t n_items, void *k_pool,
+                                         void *v_pool, int64_t num_pool_blocks, int32_t head_size,
+                                         int32_t block_size, int32_t dtype, void *stream);
+
 /* ---- Operators of the model step around the attention layer ---------------
  * The reference's LLaMA layer takes RMSNorm and SiluAndMul from its vLLM fork
  * (muxserve/flexserver/models/llama.py:35-36; used at :79-81, 200-203, 217-232,

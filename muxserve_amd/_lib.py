@@ -117,11 +117,22 @@ class MuxDecodeItem(ctypes.Structure):
     ]
 
 
+class MuxCacheWriteItem(ctypes.Structure):
+    _fields_ = [
+        ("positions", c_vp), ("q", c_vp), ("q_row_stride", c_i64),
+        ("k", c_vp), ("v", c_vp), ("kv_row_stride", c_i64),
+        ("cos_sin", c_vp), ("slot_mapping", c_vp),
+        ("max_position", c_i32), ("rotary_dim", c_i32), ("layer", c_i32), ("num_layers", c_i32),
+        ("num_tokens", c_i32), ("num_q_heads", c_i32), ("num_kv_heads", c_i32),
+    ]
+
+
 ATTN_SIGNATURES = {
     "mux_attn_version": (c_i32, []),
     "mux_last_hip_error": (c_i32, []),
     "mux_reshape_and_cache": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i32, c_i32,
                                       c_i32, c_i32, c_i32, c_i32, c_i32, c_vp]),
+    "mux_multi_rope_reshape_and_cache": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_vp]),
     "mux_paged_decode_workspace_bytes": (c_sz, [c_vp, c_i32, c_i32]),
     "mux_paged_decode_workspace_init": (c_i32, [c_vp, c_sz, c_vp]),
     "mux_multi_decode": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_i32,

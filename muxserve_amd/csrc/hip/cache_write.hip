@@ -95,11 +95,13 @@ constexpr int kBack = 16;                // tokens before the nominal 16 that a 
 constexpr int kSlotWin = 48;             // slots of tokens 16w-16 .. 16w+31 are examined
 constexpr int kTileRows = 32;            // a window lies inside tokens 16w-16 .. 16w+15
 
+// One workgroup's window: kv head h, tokens around T0 (a multiple of 16).
 template <typename T, bool ROPE>
-__global__ __launch_bounds__(256) void reshape_and_cache_kernel(
+__device__ __forceinline__ void cache_write_window(
     uint16_t *k, const uint16_t *__restrict__ v, int64_t row_stride,
     uint4 *__restrict__ k_pool, uint16_t *__restrict__ v_pool, int64_t num_blocks,
-    const int64_t *__restrict__ slots, int64_t slot_stride, int num_tokens, int block_size, const RopeArgs R) {
+    const int64_t *__restrict__ slots, int64_t slot_stride, int num_tokens, int block_size, const RopeArgs &R,
+    const int h, const int T0) {
   constexpr int D = kHeadSize;
   __shared__ __attribute__((aligned(16))) uint16_t kt[kTileRows][kVtRow];
   __shared__ __attribute__((aligned(16))) uint16_t vt[kTileRows][kVtRow];
@@ -107,11 +109,6 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
   const int lane = threadIdx.x & 63;
   const int i = threadIdx.x & 15;
   const int c = threadIdx.x >> 4;
-  // Heads vary fastest over the workgroup ids: workgroups that run together read
-  // the neighbouring 256-byte head slices of the same k/v rows (one DRAM page)
-  // rather than one slice out of each of many rows.
-  const int h = blockIdx.x;
-  const int T0 = blockIdx.y * 16;
   const int64_t pool_slots = num_blocks * block_size;
 
   // Slots of tokens T0-16 .. T0+31 (bit j of the masks below is token T0-16+j);
@@ -278,6 +275,57 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
   }
 }
 
+// Heads vary fastest over the workgroup ids: workgroups that run together read
+// the neighbouring 256-byte head slices of the same k/v rows (one DRAM page)
+// rather than one slice out of each of many rows.
+template <typename T, bool ROPE>
+__global__ __launch_bounds__(256) void reshape_and_cache_kernel(
+    uint16_t *k, const uint16_t *__restrict__ v, int64_t row_stride,
+    uint4 *__restrict__ k_pool, uint16_t *__restrict__ v_pool, int64_t num_blocks,
+    const int64_t *__restrict__ slots, int64_t slot_stride, int num_tokens, int block_size, const RopeArgs R) {
+  cache_write_window<T, ROPE>(k, v, row_stride, k_pool, v_pool, num_blocks, slots, slot_stride, num_tokens,
+                              block_size, R, blockIdx.x, blockIdx.y * 16);
+}
+
+// Several colocated models' cache writes of one step in one grid: the kernel
+// argument carries one descriptor per model, a workgroup finds its model from
+// the models' first workgroup ids and then does what the single-model kernel
+// does (heads fastest within a model).
+struct CacheWriteItemDev {
+  uint16_t *k;
+  const uint16_t *v;
+  int64_t row_stride;
+  const int64_t *slots;          // layer slice of the model's slot mapping
+  int64_t slot_stride;
+  RopeArgs rope;
+  int32_t num_tokens;
+  int32_t num_kv_heads;
+  int32_t work_begin;            // first workgroup of this model
+};
+struct MultiCacheWriteParams {
+  CacheWriteItemDev it[MUXA_MAX_DECODE_ITEMS];
+  uint4 *k_pool;
+  uint16_t *v_pool;
+  int64_t num_blocks;
+  int32_t n_items;
+  int32_t block_size;
+};
+
+template <typename T, bool ROPE>
+__global__ __launch_bounds__(256) void multi_reshape_and_cache_kernel(const MultiCacheWriteParams P) {
+  const int w = blockIdx.x;
+  int ii = 0;
+#pragma unroll
+  for (int i = 1; i < MUXA_MAX_DECODE_ITEMS; ++i)
+    if (i < P.n_items && w >= P.it[i].work_begin) ii = i;
+  const CacheWriteItemDev I = P.it[ii];
+  const int local = w - I.work_begin;
+  const int ty = local / I.num_kv_heads;
+  const int h = local - ty * I.num_kv_heads;
+  cache_write_window<T, ROPE>(I.k, I.v, I.row_stride, P.k_pool, P.v_pool, P.num_blocks, I.slots, I.slot_stride,
+                              I.num_tokens, P.block_size, I.rope, h, ty * 16);
+}
+
 }  // namespace mux
 
 namespace mux {
@@ -368,6 +416,76 @@ extern "C" int32_t mux_rope_reshape_and_cache(const int64_t *positions, void *q,
     hipLaunchKernelGGL((reshape_and_cache_kernel<BF16, true>), grid, dim3(256), 0, st, static_cast<uint16_t *>(k),
                        static_cast<const uint16_t *>(v), kv_row_stride, static_cast<uint4 *>(k_pool),
                        static_cast<uint16_t *>(v_pool), num_pool_blocks, slots, slot_stride, num_tokens, block_size, R);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(e);
+  return MUXA_OK;
+}
+
+extern "C" int32_t mux_multi_rope_reshape_and_cache(const MuxCacheWriteItem *items, int32_t n_items, void *k_pool,
+                                                    void *v_pool, int64_t num_pool_blocks, int32_t head_size,
+                                                    int32_t block_size, int32_t dtype, void *stream) {
+  using namespace mux;
+  if (!items || n_items <= 0 || n_items > MUXA_MAX_DECODE_ITEMS) return MUXA_EINVAL;
+  MultiCacheWriteParams P = {};
+  P.k_pool = static_cast<uint4 *>(k_pool);
+  P.v_pool = static_cast<uint16_t *>(v_pool);
+  P.num_blocks = num_pool_blocks;
+  P.block_size = block_size;
+  // Either every model of the call that has tokens rotates (positions given) or none does.
+  bool rope = false;
+  for (int i = 0; i < n_items; ++i)
+    if (items[i].num_tokens > 0) {
+      rope = items[i].positions != nullptr;
+      break;
+    }
+  int64_t work = 0;
+  for (int i = 0; i < n_items; ++i) {
+    const MuxCacheWriteItem &it = items[i];
+    const int32_t rc = check_cache_write(it.k, it.v, it.kv_row_stride, k_pool, v_pool, num_pool_blocks,
+                                         it.slot_mapping, it.layer, it.num_layers, it.num_tokens, it.num_kv_heads,
+                                         head_size, block_size, dtype);
+    if (rc != MUXA_OK) return rc;
+    if (it.num_tokens > 0 && (it.positions != nullptr) != rope) return MUXA_EINVAL;
+    RopeArgs R{};
+    if (rope && it.num_tokens > 0) {
+      if ((it.num_tokens > 0 && !it.cos_sin) || it.max_position <= 0) return MUXA_EINVAL;
+      if (it.rotary_dim != kHeadSize) return MUXA_EUNSUPPORTED;
+      if (it.q != nullptr) {
+        if (it.num_q_heads <= 0 || it.num_q_heads % it.num_kv_heads != 0) return MUXA_EINVAL;
+        if (it.q_row_stride < static_cast<int64_t>(it.num_q_heads) * kHeadSize || it.q_row_stride % 8 != 0)
+          return MUXA_EINVAL;
+        if (reinterpret_cast<uintptr_t>(it.q) & 15u) return MUXA_EINVAL;
+      }
+      R.q = static_cast<uint16_t *>(it.q);
+      R.q_stride = it.q_row_stride;
+      R.ratio = it.q ? it.num_q_heads / it.num_kv_heads : 0;
+      R.positions = it.positions;
+      R.cos_sin = it.cos_sin;
+      R.max_position = it.max_position;
+    }
+    if (it.num_tokens == 0) continue;
+    CacheWriteItemDev &d = P.it[P.n_items++];
+    d.k = static_cast<uint16_t *>(it.k);
+    d.v = static_cast<const uint16_t *>(it.v);
+    d.row_stride = it.kv_row_stride;
+    d.slots = it.slot_mapping + static_cast<int64_t>(it.layer) * it.num_kv_heads;
+    d.slot_stride = static_cast<int64_t>(it.num_layers) * it.num_kv_heads;
+    d.rope = R;
+    d.num_tokens = it.num_tokens;
+    d.num_kv_heads = it.num_kv_heads;
+    d.work_begin = static_cast<int32_t>(work);
+    work += static_cast<int64_t>((it.num_tokens + 15) / 16) * it.num_kv_heads;
+    if (work > 0x7fffffff) return MUXA_EUNSUPPORTED;
+  }
+  if (P.n_items == 0) return MUXA_OK;
+  const dim3 grid(static_cast<unsigned>(work));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!rope)
+    hipLaunchKernelGGL((multi_reshape_and_cache_kernel<F16, false>), grid, dim3(256), 0, st, P);
+  else if (dtype == MUXA_DTYPE_F16)
+    hipLaunchKernelGGL((multi_reshape_and_cache_kernel<F16, true>), grid, dim3(256), 0, st, P);
+  else
+    hipLaunchKernelGGL((multi_reshape_and_cache_kernel<BF16, true>), grid, dim3(256), 0, st, P);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(e);
   return MUXA_OK;

@@ -301,6 +301,79 @@ def rope_reshape_and_cache(positions: torch.Tensor, q: Optional[torch.Tensor], k
     _lib.check_attn(rc, "mux_rope_reshape_and_cache")
 
 
+@dataclass
+class CacheWriteCall:
+    """One model's cache write of a step (an element of a fused launch).  With
+    positions and cos_sin the write rotates q and k in place first (rotary_dim
+    = 128); without, it is the plain scatter."""
+    k: torch.Tensor                       # [>=T, Hkv*128]
+    v: torch.Tensor
+    slot_mapping: torch.Tensor            # int64 [T, L, Hkv]
+    layer: int = 0
+    positions: Optional[torch.Tensor] = None     # int64 [>=T]
+    cos_sin: Optional[torch.Tensor] = None       # float32 [max_position, 128]
+    q: Optional[torch.Tensor] = None             # [>=T, Hq*128]
+    num_tokens: Optional[int] = None
+
+    def to_item(self, pool_dtype) -> _lib.MuxCacheWriteItem:
+        k, v, sm = self.k, self.v, self.slot_mapping
+        _need_cuda(k, v, sm)
+        if sm.dtype != torch.int64 or sm.dim() != 3 or not sm.is_contiguous():
+            raise ValueError("slot_mapping: expected contiguous int64 [T, L, Hkv]")
+        T, L, H = sm.shape
+        if self.num_tokens is not None:
+            T = min(T, int(self.num_tokens))
+        stride = _rows(k, "k")
+        if _rows(v, "v") != stride or k.shape != v.shape or k.dtype != v.dtype or k.dtype != pool_dtype:
+            raise ValueError("k and v must have the same shape, strides and dtype as each other and the pool's dtype")
+        if k.shape[0] < T or k.shape[1] != H * HEAD_SIZE:
+            raise ValueError(f"k: expected [>={T}, {H * HEAD_SIZE}], got {tuple(k.shape)}")
+        it = _lib.MuxCacheWriteItem()
+        it.k, it.v, it.kv_row_stride = k.data_ptr(), v.data_ptr(), stride
+        it.slot_mapping, it.layer, it.num_layers, it.num_tokens, it.num_kv_heads = sm.data_ptr(), int(self.layer), L, T, H
+        if self.positions is not None:
+            pos, cs = self.positions, self.cos_sin
+            if cs is None:
+                raise ValueError("positions without cos_sin")
+            _need_cuda(pos, cs)
+            if pos.dtype != torch.int64 or pos.dim() != 1 or not pos.is_contiguous() or pos.shape[0] < T:
+                raise ValueError("positions: expected contiguous int64 [>=T]")
+            if cs.dtype != torch.float32 or cs.dim() != 2 or not cs.is_contiguous():
+                raise ValueError("cos_sin: expected contiguous float32 [max_position, rotary_dim]")
+            it.positions, it.cos_sin = pos.data_ptr(), cs.data_ptr()
+            it.max_position, it.rotary_dim = cs.shape[0], cs.shape[1]
+            if self.q is not None:
+                q = self.q
+                _need_cuda(q)
+                if q.dtype != k.dtype or q.shape[1] % HEAD_SIZE or q.shape[0] < T:
+                    raise ValueError("q [>=T, Hq*128] of the dtype of k expected")
+                it.q, it.q_row_stride, it.num_q_heads = q.data_ptr(), _rows(q, "q"), q.shape[1] // HEAD_SIZE
+        return it
+
+
+def cache_write_items(calls: List[CacheWriteCall], pool_dtype):
+    """The checked descriptor array of a fused cache write.  A loop that issues
+    the same write again and again (same tensors) may build it once and pass it
+    to multi_reshape_and_cache in place of the calls; the tensors must stay alive."""
+    return (_lib.MuxCacheWriteItem * len(calls))(*[c.to_item(pool_dtype) for c in calls])
+
+
+def multi_reshape_and_cache(calls, k_pool: torch.Tensor, v_pool: torch.Tensor, stream=None) -> None:
+    """The cache writes (fused with the rotary embedding when the calls carry
+    positions) of several colocated models' step in one launch; bit-identical
+    to one reshape_and_cache / rope_reshape_and_cache call per model.  `calls`:
+    a list of CacheWriteCall or the array cache_write_items made from one."""
+    if not 1 <= len(calls) <= _lib.MUXA_MAX_DECODE_ITEMS:
+        raise ValueError(f"1..{_lib.MUXA_MAX_DECODE_ITEMS} models per launch")
+    _need_cuda(k_pool, v_pool)
+    bs = _check_pools(k_pool, v_pool)
+    items = calls if isinstance(calls, ctypes.Array) else cache_write_items(calls, k_pool.dtype)
+    rc = _lib.attn().mux_multi_rope_reshape_and_cache(ctypes.addressof(items), len(calls), k_pool.data_ptr(),
+                                                      v_pool.data_ptr(), k_pool.shape[0], HEAD_SIZE, bs,
+                                                      _dtype_code(k_pool), _stream_ptr(stream))
+    _lib.check_attn(rc, "mux_multi_rope_reshape_and_cache")
+
+
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None,
              num_tokens: Optional[int] = None, stream=None) -> torch.Tensor:
     """out[t] = T(x[t] * rsqrt(mean(x[t]^2) + eps)) * weight for x [T, hidden]."""

@@ -569,6 +569,49 @@ def test_gather_read_probe_runs_and_rejects_what_it_cannot_read():
                                              None) == -1      # invalid argument
 
 
+def test_split_context_hand_off_is_stable_over_two_thousand_launches():
+    """The hand-off of split contexts between workgroups (partial results
+    published with device-coherent stores, one arrival counter per sequence and
+    head group, the last arriver combines): 2000 launches of a split-heavy batch
+    - partitions of 64 tokens, contexts 65..2048, so up to 32 partitions meet per
+    head - alternating between two workspaces, every output compared bitwise
+    with the first launch's.  The comparison stays on the device and is read
+    back every 100 launches; the run stops at the first mismatch."""
+    _announce("decode split hand-off, 2000 launches")
+    bs, Hq, B = 16, 8, 48
+    rng = np.random.Generator(np.random.PCG64(77))
+    ctx = rng.integers(65, 2049, size=B).astype(np.int32)
+    ctx[:4] = [65, 2048, 128, 1999]
+    need = int(((ctx + bs - 1) // bs).sum()) * Hq
+    N = need + 64
+    bt, _ = workloads.build_tables(ctx, Hq, bs, rng.permutation(N)[:need])
+    m = workloads.DecodeModel("m", Hq, Hq, ctx, bt)
+    dk, dv = allocate_gpu_cache(N, bs, DEV)
+    workloads.fill_blocks(dk, dv, m.used_blocks(bs), seed=3)
+    m.to_device(DEV, torch.float16, seed=4)
+    lib_need = (B * Hq * 32) * (128 + 2) * 4 + (2 << 20)
+    spaces = [torch.zeros((lib_need,), dtype=torch.uint8, device=DEV) for _ in range(2)]
+    host_lens = torch.from_numpy(ctx)
+
+    def launch(i):
+        ops.paged_decode(m.out, m.q, dk, dv, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                         partition_size=64, workspace=spaces[i % 2],
+                         context_lens_host=host_lens if (i // 2) % 2 else None)
+
+    launch(0)
+    torch.cuda.synchronize()
+    first = m.out.clone()
+    want = orc.paged_decode(m.q.cpu(), dk.cpu(), dv.cpu(), torch.from_numpy(bt), ctx, m.scale)
+    _check(first[:B].float().cpu(), want)
+    bad = torch.zeros((), dtype=torch.int32, device=DEV)
+    for i in range(1, 2001):
+        m.out.zero_()
+        launch(i)
+        bad += (m.out != first).any().to(torch.int32)
+        if i % 100 == 0:
+            assert int(bad.item()) == 0, f"a launch among {i - 99}..{i} differs from the first"
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_decode_random_shapes_against_the_oracle(seed):
     """Seeded draws over head grouping, block size, storage type, partition size,

@@ -158,6 +158,87 @@ def test_fused_rotary_cache_write_equals_the_two_kernels(dtype, Hq, Hkv, bs):
     assert torch.equal(results[1][0][T:], qkv.cpu().view(torch.int16)[T:]), "padding rows must not be touched"
 
 
+@pytest.mark.parametrize("rope", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_multi_model_cache_write_equals_one_launch_per_model(rope, dtype):
+    """mux_multi_rope_reshape_and_cache over three colocated models (7B, 13B, a
+    grouped-query shape; a decode-shaped step of single tokens for two of them
+    and packed ragged prompts for the third, one empty model in between) against
+    one call per model: q, k rows and both pools bitwise equal, and the plain
+    variant bitwise equal to the oracle's scatter."""
+    print(f"[case] multi-model cache write rope={rope} {dtype}", flush=True)
+    from oracle import attn_oracle as orc
+    from muxserve_amd import workloads
+    from muxserve_amd.attention import build_cos_sin_cache
+    from muxserve_amd.pool import allocate_gpu_cache
+    bs, L, layer = 16, 2, 1
+    rng = np.random.Generator(np.random.PCG64(91))
+    g = torch.Generator().manual_seed(91)
+    shapes = [(32, 32, 32), (40, 40, 16), (8, 2, 0), (16, 4, None)]      # Hq, Hkv, decode tokens (None: prompts)
+    lens3 = rng.permutation(np.arange(1, 24)).astype(np.int32)
+    need = sum(hk * (t if t is not None else int(((lens3 + bs - 1) // bs).sum())) for _, hk, t in shapes)
+    N = need + 11
+    ids = rng.permutation(N)
+    cos_sin = build_cos_sin_cache(D, 4096, 10000.0, DEV)
+    models, cur = [], 0
+    for hq, hk, t in shapes:
+        if t is None:
+            slots1, used = workloads.prefill_slot_mapping(lens3, hk, bs, ids[cur:])
+            T = int(lens3.sum())
+        else:
+            # a decode step: every sequence writes one token somewhere inside its last block
+            T = t
+            blk = ids[cur:cur + T * hk].reshape(T, hk).astype(np.int64)
+            slots1 = (blk * bs + rng.integers(0, bs, size=(T, 1)))[:, None, :]
+            used = T * hk
+        cur += used
+        slots = np.full((T, L, hk), -1, dtype=np.int64)
+        slots[:, layer, :] = slots1[:, 0, :]
+        if T > 3:
+            slots[2, layer, 0] = -1
+        pad = (T + 7) // 8 * 8
+        qkv = torch.randn((pad, (hq + 2 * hk) * D), generator=g).to(dtype).to(DEV)
+        pos = torch.from_numpy(rng.integers(0, 4096, size=pad)).to(DEV)
+        models.append((hq, hk, T, qkv, pos, torch.from_numpy(slots).to(DEV), slots))
+    results = []
+    for fused in (False, True):
+        kp, vp = allocate_gpu_cache(N, bs, DEV, dtype=dtype)
+        kp.zero_()
+        vp.zero_()
+        xs, calls = [], []
+        for hq, hk, T, qkv, pos, dslots, _ in models:
+            x = qkv.clone()
+            xs.append(x)
+            q, k, v = x.split([hq * D, hk * D, hk * D], dim=-1)
+            if fused:
+                calls.append(ops.CacheWriteCall(k, v, dslots, layer=layer, positions=pos if rope else None,
+                                                cos_sin=cos_sin if rope else None, q=q if rope else None,
+                                                num_tokens=T))
+            elif rope:
+                ops.rope_reshape_and_cache(pos, q, k, v, cos_sin, kp, vp, dslots, layer=layer, num_tokens=T)
+            else:
+                ops.reshape_and_cache(k, v, kp, vp, dslots, layer=layer, num_tokens=T)
+        if fused:
+            ops.multi_reshape_and_cache(calls, kp, vp)
+        torch.cuda.synchronize()
+        results.append(([x.cpu().view(torch.int16) for x in xs], kp.cpu(), vp.cpu()))
+    for xa, xb in zip(results[0][0], results[1][0]):
+        assert torch.equal(xa, xb), "q/k rows differ between the fused launch and the per-model launches"
+    assert torch.equal(results[0][1].view(torch.int16), results[1][1].view(torch.int16))
+    assert torch.equal(results[0][2].view(torch.int16), results[1][2].view(torch.int16))
+    if not rope:
+        hk_pool, hv_pool = orc.allocate_pool(N, bs, dtype)
+        hk_pool.zero_()
+        hv_pool.zero_()
+        for hq, hk, T, qkv, pos, _, slots in models:
+            if T == 0:
+                continue
+            _, k, v = qkv.cpu().split([hq * D, hk * D, hk * D], dim=-1)
+            orc.reshape_and_cache(k[:T], v[:T], hk_pool, hv_pool, torch.from_numpy(slots), layer=layer)
+        assert torch.equal(results[1][1].view(torch.int16), hk_pool.view(torch.int16))
+        assert torch.equal(results[1][2].view(torch.int16), hv_pool.view(torch.int16))
+
+
 def test_empty_steps_are_accepted():
     """No tokens, no sequences, no prompts, no sampled rows: every entry point
     returns without launching and without touching its outputs."""
