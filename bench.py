@@ -60,7 +60,8 @@ def parse():
                     help="prefill3: do not pass the host-side prompt lengths (grid sized by the longest prompt)")
     ap.add_argument("--unfused", action="store_true", help="one launch per model instead of one fused launch")
     ap.add_argument("--workload", default="mixed3_decode",
-                    choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long", "model_ops", "host_step"],
+                    choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long", "model_ops", "host_step",
+                             "cu_masks"],
                     help="mixed3_decode is the headline metric; the others are the remaining synthetic "
                          "shapes, each printing its own JSON line")
     return ap.parse_args()
@@ -336,6 +337,40 @@ def bench_colocated(args):
                  "tokens/s", args, res["decode_concurrent_ms"], res, roof)
 
 
+def bench_cu_masks(args):
+    """Where CU-masked streams run: for a set of masks, the compute units the
+    workgroups of a recording kernel were started on (accelerator die, shader
+    engine, compute unit from the XCC_ID / HW_ID registers), per die."""
+    import torch
+    from muxserve_amd import ops, workloads
+    ncu, nxcd = ops.device_cu_info()
+    rows = {}
+
+    def record(name, stream):
+        where = workloads.where_workgroups_run(stream)
+        per_die = np.bincount([w[0] for w in where], minlength=nxcd).tolist()
+        per_se = np.bincount([w[1] for w in where], minlength=4).tolist()
+        rows[name] = {"compute_units": len(where), "per_die": per_die, "per_shader_engine": per_se,
+                      "first": [list(w) for w in where[:6]]}
+        return set(where)
+
+    sets = {}
+    for name, kw in (("percent 0-40", dict(lo_percent=0, hi_percent=40)), ("percent 40-100", dict(lo_percent=40, hi_percent=100)),
+                     ("parts {0}", dict(parts=[0])), ("parts {9}", dict(parts=[9])), ("parts {0,3,7}", dict(parts=[0, 3, 7])),
+                     ("parts {1,2,9}", dict(parts=[1, 2, 9])), ("parts {4,5,6,8}", dict(parts=[4, 5, 6, 8]))):
+        st = ops.CUMaskedStream(**kw)
+        sets[name] = record(name, st)
+        st.close()
+    sets["no mask"] = record("no mask", None)
+    names = list(sets)
+    overlaps = {f"{a} & {b}": len(sets[a] & sets[b]) for i, a in enumerate(names) for b in names[i + 1:]
+                if a != "no mask" and b != "no mask"}
+    cfg = {"workload": "cu_masks", "num_cus": ncu, "num_dies": nxcd, "masks": rows, "shared_compute_units": overlaps}
+    return _line("compute units reached through CU-masked streams", float(ncu), "compute units", args, 0.0, cfg,
+                 {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": None, "traffic": None,
+                  "kernel": "probe_where_kernel (records XCC_ID / HW_ID per workgroup)"}, dtype="u32")
+
+
 def bench_gqa_long(args):
     """Config 5: 64 query heads over 8 kv heads, bf16, batch 64, ctx U[2048, 8192]."""
     import torch
@@ -606,7 +641,7 @@ def main():
         print("bench.py: this build runs on one GPU only (no collectives or sharding); use --gpus 1",
               file=sys.stderr)
         sys.exit(2)
-    other = {"prefill3": bench_prefill3, "cache_write": bench_cache_write, "colocated": bench_colocated,
+    other = {"prefill3": bench_prefill3, "cache_write": bench_cache_write, "colocated": bench_colocated, "cu_masks": bench_cu_masks,
              "gqa_long": bench_gqa_long, "model_ops": bench_model_ops, "host_step": bench_host_step}
     if args.workload in other:
         print(json.dumps(other[args.workload](args)))

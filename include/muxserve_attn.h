@@ -347,6 +347,21 @@ int32_t mux_build_step_inputs(int32_t *mirror, int32_t max_rows, int32_t max_blo
  * hipStream_t; *num_cus_out (optional) the number of CUs enabled. */
 int32_t mux_stream_create_cu_range(void **stream_out, int32_t lo_percent, int32_t hi_percent,
                                    int32_t *num_cus_out);
+/* The same for a SET of tenths of the GPU: the reference's scheduler hands out
+ * compute in 10 parts (SMResource, muxserve/muxsched/resource.py:35-81) and a
+ * job holds whichever parts were free - not a contiguous range.  Bit p of
+ * part_mask (p = 0..9) enables mask bits [N*p/10, N*(p+1)/10) of the device's N
+ * compute units.  Consecutive mask bits go round-robin over the accelerator
+ * dies first and the shader engines next (measured on MI355X with a kernel that
+ * records XCC_ID / HW_ID per workgroup), so every part takes 3 or 4 compute
+ * units from each of the 8 dies, two part sets without a common part never share
+ * a compute unit, and no die is left without one (the driver refuses such
+ * masks).  mux_cu_parts_mask builds the mask words on the host without a GPU
+ * (words: n_words >= ceil(num_cus / 32) uint32) and returns the number of
+ * compute units enabled, or a negative code. */
+#define MUXA_CU_PARTS 10
+int32_t mux_cu_parts_mask(uint32_t part_mask, int32_t num_cus, uint32_t *words, int32_t n_words);
+int32_t mux_stream_create_cu_parts(void **stream_out, uint32_t part_mask, int32_t *num_cus_out);
 int32_t mux_stream_destroy(void *stream);
 /* Device facts used by the mask builder: out = [num_cus, num_xcds]. */
 int32_t mux_device_cu_info(int32_t out[2]);

@@ -156,6 +156,8 @@ ATTN_SIGNATURES = {
                                   c_vp, c_sz, c_vp]),
     "mux_build_step_inputs": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_i32, c_vp, c_i64, c_i32,
                                       c_i32, c_vp, c_vp, c_i32, c_vp]),
+    "mux_cu_parts_mask": (c_i32, [ctypes.c_uint32, c_i32, c_vp, c_i32]),
+    "mux_stream_create_cu_parts": (c_i32, [c_vp, ctypes.c_uint32, c_vp]),
     "mux_stream_create_cu_range": (c_i32, [c_vp, c_i32, c_i32, c_vp]),
     "mux_stream_destroy": (c_i32, [c_vp]),
     "mux_device_cu_info": (c_i32, [c_vp]),
@@ -184,6 +186,8 @@ def probe():
         lib = _open(PROBE_LIB_PATH)
         lib.mux_probe_gather_read.restype = c_i32
         lib.mux_probe_gather_read.argtypes = [c_vp, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp]
+        lib.mux_probe_where.restype = c_i32
+        lib.mux_probe_where.argtypes = [c_vp, c_i32, c_i32, c_vp]
         _probe = lib
     return _probe
 

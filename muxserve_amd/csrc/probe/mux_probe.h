@@ -23,6 +23,14 @@ int32_t mux_probe_gather_read(const void *k_pool, const void *v_pool, int64_t nu
                               const int32_t *block_ids, int64_t n_blocks, int32_t block_size,
                               uint32_t *sink, void *stream);
 
+/* Records where the workgroups of a launch run: out (DEVICE uint32
+ * [num_workgroups, 2]) receives per workgroup the XCC_ID register (accelerator
+ * die in its low 4 bits) and the HW_ID register (compute unit id in bits 8-11,
+ * shader array in bit 12, shader engine in bits 13-15) of its compute unit; each
+ * workgroup (one wave) then idles for spin_microseconds so that the launch
+ * spreads over every compute unit its stream may use. */
+int32_t mux_probe_where(uint32_t *out, int32_t num_workgroups, int32_t spin_microseconds, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -65,3 +65,34 @@ extern "C" int32_t mux_probe_gather_read(const void *k_pool, const void *v_pool,
                      static_cast<const uint4 *>(v_pool), block_ids, n_blocks, num_pool_blocks, sink);
   return hipGetLastError() == hipSuccess ? 0 : -4;
 }
+
+// ---------------------------------------------------------------------------
+// Where workgroups run: every workgroup of the launch records the accelerator
+// die (XCC_ID register) and the hardware id word (HW_ID register: compute unit,
+// shader array, shader engine, ...) of the compute unit it was started on, then
+// spins for `spin_ticks` of the 100 MHz clock so that the launch spreads over
+// every compute unit the stream may use.  The evidence behind CU-masked streams:
+// which mask bit enables which compute unit.
+// ---------------------------------------------------------------------------
+namespace mux {
+
+__global__ __launch_bounds__(64) void probe_where_kernel(uint32_t *out, int spin_ticks) {
+  // s_getreg_b32: id | offset << 6 | (size - 1) << 11; HW_ID is register 4, XCC_ID register 20.
+  const uint32_t hw_id = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (31 << 11));
+  const uint32_t xcc_id = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (31 << 11));
+  if (threadIdx.x == 0) {
+    out[2 * blockIdx.x] = xcc_id;
+    out[2 * blockIdx.x + 1] = hw_id;
+  }
+  const long long until = static_cast<long long>(__builtin_amdgcn_s_memrealtime()) + spin_ticks;
+  while (static_cast<long long>(__builtin_amdgcn_s_memrealtime()) < until) __builtin_amdgcn_s_sleep(8);
+}
+
+}  // namespace mux
+
+extern "C" int32_t mux_probe_where(uint32_t *out, int32_t num_workgroups, int32_t spin_microseconds, void *stream) {
+  if (!out || num_workgroups <= 0 || spin_microseconds < 0 || spin_microseconds > 100000) return -1;
+  hipLaunchKernelGGL(mux::probe_where_kernel, dim3(static_cast<uint32_t>(num_workgroups)), dim3(64), 0,
+                     static_cast<hipStream_t>(stream), out, spin_microseconds * 100);
+  return hipGetLastError() == hipSuccess ? 0 : -4;
+}

@@ -459,15 +459,29 @@ class CUMaskedStream:
     replacement for a per-process MPS percentage).  Usable wherever a stream is
     accepted: ``with torch.cuda.stream(s.torch_stream): ...`` or ``stream=s``."""
 
-    def __init__(self, lo_percent: int, hi_percent: int):
+    def __init__(self, lo_percent: Optional[int] = None, hi_percent: Optional[int] = None, parts=None):
+        """Either a percent range [lo_percent, hi_percent) of the compute-unit
+        mask, or `parts`: the tenths of the GPU a job holds (ids 0..9 in any
+        combination, as muxserve_amd.cu_resource.CUResource hands them out)."""
         import ctypes as _c
         handle = _c.c_void_p()
         ncu = _c.c_int32()
-        rc = _lib.attn().mux_stream_create_cu_range(_c.byref(handle), int(lo_percent), int(hi_percent), _c.byref(ncu))
-        _lib.check_attn(rc, "mux_stream_create_cu_range")
+        if parts is not None:
+            if lo_percent is not None or hi_percent is not None:
+                raise ValueError("give a percent range or a set of parts, not both")
+            from .cu_resource import part_bits
+            self.part_mask = part_bits(parts)
+            rc = _lib.attn().mux_stream_create_cu_parts(_c.byref(handle), self.part_mask, _c.byref(ncu))
+            _lib.check_attn(rc, "mux_stream_create_cu_parts")
+            self.lo_percent = self.hi_percent = None
+        else:
+            rc = _lib.attn().mux_stream_create_cu_range(_c.byref(handle), int(lo_percent), int(hi_percent),
+                                                        _c.byref(ncu))
+            _lib.check_attn(rc, "mux_stream_create_cu_range")
+            self.lo_percent, self.hi_percent = int(lo_percent), int(hi_percent)
+            self.part_mask = None
         self.cuda_stream = handle.value
         self.num_cus = ncu.value
-        self.lo_percent, self.hi_percent = int(lo_percent), int(hi_percent)
         self.torch_stream = torch.cuda.ExternalStream(self.cuda_stream)
 
     def synchronize(self):

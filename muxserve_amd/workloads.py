@@ -260,3 +260,21 @@ def probe_gather_read(k_pool: torch.Tensor, v_pool: torch.Tensor, block_ids: tor
                                             block_ids.data_ptr(), block_ids.numel(), bs, sink.data_ptr(),
                                             ops._stream_ptr(stream))
     _lib.check_attn(rc, "mux_probe_gather_read")
+
+
+def where_workgroups_run(stream=None, num_workgroups: int = 8192, spin_microseconds: int = 20, device="cuda:0"):
+    """Measuring aid (libmuxprobe.so): launches single-wave workgroups that idle
+    for spin_microseconds on `stream` and returns the sorted set of compute units
+    they ran on as (accelerator die, shader engine, shader array, compute unit)
+    tuples, read from the XCC_ID and HW_ID registers."""
+    from . import _lib, ops
+    out = torch.zeros((num_workgroups, 2), dtype=torch.int32, device=device)
+    torch.cuda.synchronize()
+    rc = _lib.probe().mux_probe_where(out.data_ptr(), int(num_workgroups), int(spin_microseconds),
+                                      ops._stream_ptr(stream))
+    _lib.check_attn(rc, "mux_probe_where")
+    torch.cuda.synchronize()
+    o = out.cpu().numpy().astype(np.uint32)
+    xcc, hw = o[:, 0] & 0xf, o[:, 1]
+    return sorted(set(zip(xcc.tolist(), ((hw >> 13) & 7).tolist(), ((hw >> 12) & 1).tolist(),
+                          ((hw >> 8) & 0xf).tolist())))

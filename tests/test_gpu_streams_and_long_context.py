@@ -56,6 +56,48 @@ def test_cu_masked_streams_run_prefill_and_decode_concurrently_and_correctly():
         ops.CUMaskedStream(50, 50)
 
 
+def test_part_set_streams_run_on_disjoint_compute_units_spread_over_every_die():
+    """Streams made from sets of tenths of the GPU (what the scheduler's part
+    bookkeeping hands out: any combination, not a contiguous range): the
+    compute units their workgroups really run on - read from the XCC_ID / HW_ID
+    registers by a recording kernel - are as many as the mask enables, differ
+    between streams without a common part, and take every accelerator die's
+    share within one compute unit per part."""
+    print("[case] part-set cu masks, where workgroups run", flush=True)
+    from muxserve_amd.cu_resource import CUResource
+    ncu, nxcd = ops.device_cu_info()
+    res = CUResource()
+    held_a = res.allocate(3)                      # parts 9, 8, 7
+    held_b = res.allocate(2)                      # parts 6, 5
+    res.free(held_a[1:2])                         # part 8 back
+    held_c = res.allocate(2)                      # parts 8, 4: not contiguous with each other
+    sets = {"a": [held_a[0], held_a[2]], "b": held_b, "c": held_c, "one": [0]}
+    seen = {}
+    for name, parts in sets.items():
+        st = ops.CUMaskedStream(parts=parts)
+        where = workloads.where_workgroups_run(st)
+        st.close()
+        assert len(where) == st.num_cus, (name, len(where), st.num_cus)
+        per_die = np.bincount([w[0] for w in where], minlength=nxcd)
+        assert per_die.min() >= 1 and per_die.max() - per_die.min() <= len(parts), (name, per_die)
+        seen[name] = set(where)
+    for x in seen:
+        for y in seen:
+            if x < y:
+                assert not seen[x] & seen[y], f"part sets {x} and {y} share a compute unit"
+    whole = workloads.where_workgroups_run(None, num_workgroups=16384)
+    assert len(whole) == ncu and set().union(*seen.values()) <= set(whole)
+    # the percent ranges of the colocated configuration are disjoint as well
+    s40, s60 = ops.CUMaskedStream(0, 40), ops.CUMaskedStream(40, 100)
+    w40, w60 = workloads.where_workgroups_run(s40), workloads.where_workgroups_run(s60)
+    s40.close()
+    s60.close()
+    assert not set(w40) & set(w60) and len(w40) + len(w60) == ncu
+    for w in (w40, w60):
+        per_die = np.bincount([x[0] for x in w], minlength=nxcd)
+        assert per_die.max() - per_die.min() <= 1
+
+
 def test_colocated_prefill_and_decode_at_the_benchmark_shapes():
     """The colocated configuration at its real shapes: a 30B-shaped prefill (52
     heads x 128, 4 prompts x 1024 tokens, fp16) on 40% of the compute units
