@@ -25,6 +25,7 @@ from typing import Any, Dict, List, Optional
 import torch
 
 from . import ops
+from . import torch_ops as T
 
 HEAD_SIZE = ops.HEAD_SIZE
 
@@ -155,16 +156,16 @@ class PagedAttention(torch.nn.Module):
             cache_event.wait()
         # The new tokens' K/V go into the pool first (decode reads them back).
         if key_cache is not None and value_cache is not None and n_valid > 0 and not _cache_written:
-            ops.reshape_and_cache(key, value, key_cache, value_cache, md.slot_mapping, layer=layer,
+            T.reshape_and_cache(key, value, key_cache, value_cache, md.slot_mapping, layer=layer,
                                   num_tokens=n_valid)
         if n_prompt > 0:
-            ops.prefill_causal(out[:n_prompt], query[:n_prompt], key[:n_prompt], value[:n_prompt],
+            T.prefill_causal(out[:n_prompt], query[:n_prompt], key[:n_prompt], value[:n_prompt],
                                md.cu_seqlens(query.device), md.max_prompt_len, self.scale, self.num_kv_heads,
-                               prompt_lens=md.prompt_lens_array())
+                               prompt_lens=md.prompt_lens)
         if md.num_generation_tokens > 0:
             if key_cache is None or value_cache is None:
                 raise ValueError("decode needs the KV pool")
-            ops.paged_decode(out[n_prompt:n_valid], query[n_prompt:n_valid], key_cache, value_cache,
+            T.paged_decode(out[n_prompt:n_valid], query[n_prompt:n_valid], key_cache, value_cache,
                              md.block_tables, md.context_lens, md.max_context_len, self.scale, layer=layer,
                              partition_size=self.partition_size, total_context_len=md.total_context_len,
                              context_lens_host=md.context_lens_host)
@@ -214,8 +215,8 @@ class PagedAttentionWithRoPE(PagedAttention):
             if fused:
                 if cache_event is not None:
                     cache_event.wait()
-                ops.rope_reshape_and_cache(positions, query, key, value, self._cache(query.device), key_cache,
+                T.rope_reshape_and_cache(positions, query, key, value, self._cache(query.device), key_cache,
                                            value_cache, md.slot_mapping, layer=self._layer(md), num_tokens=n_valid)
             else:
-                ops.rotary_neox(positions, query, key, self._cache(query.device), num_tokens=n_valid)
+                T.rotary_neox(positions, query, key, self._cache(query.device), num_tokens=n_valid)
         return super().forward(query, key, value, key_cache, value_cache, md, cache_event, _cache_written=fused)

@@ -111,9 +111,73 @@ void rope_reshape_and_cache(const at::Tensor &positions, at::Tensor q, at::Tenso
         "mux_rope_reshape_and_cache");
 }
 
+// The cache writes of several colocated models' step in one launch.  Element i
+// of every list describes model i; positions / qs / cos_sins are either all
+// empty (plain scatter) or one entry per model (rotary embedding of q and k in
+// place first).  num_tokens[i] < 0: all rows of slot_mappings[i].
+void multi_reshape_and_cache(at::TensorList ks, at::TensorList vs, at::Tensor k_pool, at::Tensor v_pool,
+                             at::TensorList slot_mappings, at::IntArrayRef layers, at::IntArrayRef num_tokens,
+                             at::TensorList positions, at::TensorList qs, at::TensorList cos_sins) {
+  need_gpu({&k_pool, &v_pool});
+  const int64_t bs = check_pools(k_pool, v_pool);
+  const size_t n = ks.size();
+  const bool rope = !positions.empty();
+  TORCH_CHECK(n >= 1 && n <= MUXA_MAX_DECODE_ITEMS && vs.size() == n && slot_mappings.size() == n &&
+                  layers.size() == n && num_tokens.size() == n,
+              "multi_reshape_and_cache: 1..", MUXA_MAX_DECODE_ITEMS, " models, one entry per model in every list");
+  TORCH_CHECK(rope ? (positions.size() == n && qs.size() == n && cos_sins.size() == n)
+                   : (qs.empty() && cos_sins.empty()),
+              "positions, qs and cos_sins: all empty, or one entry per model");
+  MuxCacheWriteItem items[MUXA_MAX_DECODE_ITEMS];
+  for (size_t i = 0; i < n; ++i) {
+    const at::Tensor &k = ks[i], &v = vs[i], &sm = slot_mappings[i];
+    need_gpu({&k, &v, &sm});
+    TORCH_CHECK(sm.scalar_type() == at::kLong && sm.dim() == 3 && sm.is_contiguous(),
+                "slot_mapping: expected contiguous int64 [T, L, Hkv]");
+    const int64_t T = num_tokens[i] < 0 ? sm.size(0) : std::min<int64_t>(num_tokens[i], sm.size(0));
+    const int64_t H = sm.size(2);
+    const int64_t stride = rows(k, "k");
+    TORCH_CHECK(rows(v, "v") == stride && k.sizes() == v.sizes() && k.scalar_type() == v.scalar_type() &&
+                    k.scalar_type() == k_pool.scalar_type(),
+                "k and v must have the same shape, strides and dtype as each other and the pool's dtype");
+    TORCH_CHECK(k.size(0) >= T && k.size(1) == H * kHead, "k: expected [>=T, Hkv*128]");
+    MuxCacheWriteItem &it = items[i];
+    it = MuxCacheWriteItem{};
+    it.k = k.data_ptr();
+    it.v = v.data_ptr();
+    it.kv_row_stride = stride;
+    it.slot_mapping = sm.data_ptr<int64_t>();
+    it.layer = static_cast<int32_t>(layers[i]);
+    it.num_layers = static_cast<int32_t>(sm.size(1));
+    it.num_tokens = static_cast<int32_t>(T);
+    it.num_kv_heads = static_cast<int32_t>(H);
+    if (rope) {
+      const at::Tensor &pos = positions[i], &q = qs[i], &cs = cos_sins[i];
+      need_gpu({&pos, &q, &cs});
+      TORCH_CHECK(pos.scalar_type() == at::kLong && pos.dim() == 1 && pos.is_contiguous() && pos.size(0) >= T,
+                  "positions: expected contiguous int64 [>=T]");
+      TORCH_CHECK(cs.scalar_type() == at::kFloat && cs.dim() == 2 && cs.is_contiguous(),
+                  "cos_sin: expected contiguous float32 [max_position, rotary_dim]");
+      TORCH_CHECK(q.dim() == 2 && q.scalar_type() == k.scalar_type() && q.size(0) >= T && q.size(1) % kHead == 0,
+                  "q [>=T, Hq*128] of the dtype of k expected");
+      it.positions = pos.data_ptr<int64_t>();
+      it.cos_sin = cs.data_ptr<float>();
+      it.max_position = static_cast<int32_t>(cs.size(0));
+      it.rotary_dim = static_cast<int32_t>(cs.size(1));
+      it.q = q.data_ptr();
+      it.q_row_stride = rows(q, "q");
+      it.num_q_heads = static_cast<int32_t>(q.size(1) / kHead);
+    }
+  }
+  check(mux_multi_rope_reshape_and_cache(items, static_cast<int32_t>(n), k_pool.data_ptr(), v_pool.data_ptr(),
+                                         k_pool.size(0), kHead, static_cast<int32_t>(bs), dtype_code(k_pool),
+                                         stream_of(k_pool)),
+        "mux_multi_rope_reshape_and_cache");
+}
+
 MuxDecodeItem decode_item(const at::Tensor &out, const at::Tensor &q, const at::Tensor &block_tables,
                           const at::Tensor &context_lens, int64_t max_context_len, double scale, int64_t layer,
-                          int64_t total_context_len) {
+                          int64_t total_context_len, const c10::optional<at::Tensor> &context_lens_host = c10::nullopt) {
   need_gpu({&out, &q, &block_tables, &context_lens});
   TORCH_CHECK(block_tables.scalar_type() == at::kInt && block_tables.dim() == 4 && block_tables.is_contiguous(),
               "block_tables: expected contiguous int32 [L, B, Hkv, max_blocks]");
@@ -141,6 +205,12 @@ MuxDecodeItem decode_item(const at::Tensor &out, const at::Tensor &q, const at::
   it.max_context_len = static_cast<int32_t>(max_context_len);
   it.scale = static_cast<float>(scale);
   it.context_lens_host = nullptr;
+  if (context_lens_host.has_value() && context_lens_host->defined() && context_lens_host->numel() > 0) {
+    const at::Tensor &h = *context_lens_host;
+    TORCH_CHECK(h.is_cpu() && h.scalar_type() == at::kInt && h.dim() == 1 && h.is_contiguous() && h.size(0) == B,
+                "context_lens_host: expected a contiguous CPU int32 [B] tensor");
+    it.context_lens_host = h.data_ptr<int32_t>();      // read during this call only
+  }
   return it;
 }
 
@@ -157,12 +227,13 @@ int64_t paged_decode_workspace_bytes(const at::Tensor &out, const at::Tensor &q,
 void paged_decode(at::Tensor out, const at::Tensor &q, const at::Tensor &k_pool, const at::Tensor &v_pool,
                   const at::Tensor &block_tables, const at::Tensor &context_lens, int64_t max_context_len,
                   double scale, int64_t layer, int64_t partition_size, int64_t total_context_len,
-                  at::Tensor workspace) {
+                  at::Tensor workspace, const c10::optional<at::Tensor> &context_lens_host) {
   need_gpu({&k_pool, &v_pool});
   const int64_t bs = check_pools(k_pool, v_pool);
   TORCH_CHECK(q.scalar_type() == k_pool.scalar_type(), "q dtype must equal the pool dtype");
   const MuxDecodeItem it =
-      decode_item(out, q, block_tables, context_lens, max_context_len, scale, layer, total_context_len);
+      decode_item(out, q, block_tables, context_lens, max_context_len, scale, layer, total_context_len,
+                  context_lens_host);
   void *ws = nullptr;
   size_t ws_bytes = 0;
   if (workspace.defined() && workspace.numel() > 0) {
@@ -195,19 +266,21 @@ int64_t multi_decode_workspace_bytes(at::TensorList outs, at::TensorList qs, at:
 void multi_decode(at::TensorList outs, at::TensorList qs, const at::Tensor &k_pool, const at::Tensor &v_pool,
                   at::TensorList block_tables, at::TensorList context_lens, at::IntArrayRef max_context_lens,
                   at::ArrayRef<double> scales, at::IntArrayRef layers, at::IntArrayRef total_context_lens,
-                  int64_t partition_size, at::Tensor workspace) {
+                  int64_t partition_size, at::Tensor workspace, at::TensorList context_lens_host) {
   need_gpu({&k_pool, &v_pool});
   const int64_t bs = check_pools(k_pool, v_pool);
   const size_t n = outs.size();
   TORCH_CHECK(n >= 1 && n <= MUXA_MAX_DECODE_ITEMS && qs.size() == n && block_tables.size() == n &&
                   context_lens.size() == n && max_context_lens.size() == n && scales.size() == n &&
-                  layers.size() == n && total_context_lens.size() == n,
+                  layers.size() == n && total_context_lens.size() == n &&
+                  (context_lens_host.empty() || context_lens_host.size() == n),
               "multi_decode: 1..", MUXA_MAX_DECODE_ITEMS, " models, one entry per model in every list");
   MuxDecodeItem items[MUXA_MAX_DECODE_ITEMS];
   for (size_t i = 0; i < n; ++i) {
     TORCH_CHECK(qs[i].scalar_type() == k_pool.scalar_type(), "q dtype must equal the pool dtype");
     items[i] = decode_item(outs[i], qs[i], block_tables[i], context_lens[i], max_context_lens[i], scales[i],
-                           layers[i], total_context_lens[i]);
+                           layers[i], total_context_lens[i],
+                           context_lens_host.empty() ? c10::nullopt : c10::optional<at::Tensor>(context_lens_host[i]));
   }
   void *ws = nullptr;
   size_t ws_bytes = 0;
@@ -339,18 +412,21 @@ TORCH_LIBRARY(muxserve_amd, m) {
         "int layer, int num_tokens) -> ()");
   m.def("rope_reshape_and_cache(Tensor positions, Tensor(a!) q, Tensor(b!) k, Tensor v, Tensor cos_sin, "
         "Tensor(c!) k_pool, Tensor(d!) v_pool, Tensor slot_mapping, int layer, int num_tokens) -> ()");
+  m.def("multi_reshape_and_cache(Tensor(a!)[] ks, Tensor[] vs, Tensor(b!) k_pool, Tensor(c!) v_pool, "
+        "Tensor[] slot_mappings, int[] layers, int[] num_tokens, Tensor[] positions, Tensor(d!)[] qs, "
+        "Tensor[] cos_sins) -> ()");
   m.def("paged_decode_workspace_bytes(Tensor out, Tensor q, Tensor block_tables, Tensor context_lens, "
         "int max_context_len, int partition_size) -> int");
   m.def("paged_decode(Tensor(a!) out, Tensor q, Tensor k_pool, Tensor v_pool, Tensor block_tables, "
         "Tensor context_lens, int max_context_len, float scale, int layer, int partition_size, "
-        "int total_context_len, Tensor(b!) workspace) -> ()");
+        "int total_context_len, Tensor(b!) workspace, Tensor? context_lens_host=None) -> ()");
   m.def("prefill_causal(Tensor(a!) out, Tensor q, Tensor k, Tensor v, Tensor cu_seqlens, int[] prompt_lens, "
         "int max_prompt_len, float scale, int num_kv_heads) -> ()");
   m.def("multi_decode_workspace_bytes(Tensor[] outs, Tensor[] qs, Tensor[] block_tables, Tensor[] context_lens, "
         "int[] max_context_lens, int partition_size) -> int");
   m.def("multi_decode(Tensor(a!)[] outs, Tensor[] qs, Tensor k_pool, Tensor v_pool, Tensor[] block_tables, "
         "Tensor[] context_lens, int[] max_context_lens, float[] scales, int[] layers, int[] total_context_lens, "
-        "int partition_size, Tensor(b!) workspace) -> ()");
+        "int partition_size, Tensor(b!) workspace, Tensor[] context_lens_host) -> ()");
   m.def("rotary_neox(Tensor positions, Tensor(a!) q, Tensor(b!) k, Tensor cos_sin, int num_tokens) -> ()");
   m.def("greedy_sample_workspace_bytes(int vocab_size) -> int", &greedy_sample_workspace_bytes);
   m.def("greedy_sample(Tensor embedding, Tensor hidden_states, int vocab_size, int num_rows, Tensor row_index, "
@@ -362,6 +438,7 @@ TORCH_LIBRARY(muxserve_amd, m) {
 TORCH_LIBRARY_IMPL(muxserve_amd, CUDA, m) {
   m.impl("reshape_and_cache", &reshape_and_cache);
   m.impl("rope_reshape_and_cache", &rope_reshape_and_cache);
+  m.impl("multi_reshape_and_cache", &multi_reshape_and_cache);
   m.impl("paged_decode_workspace_bytes", &paged_decode_workspace_bytes);
   m.impl("paged_decode", &paged_decode);
   m.impl("prefill_causal", &prefill_causal);

@@ -2,13 +2,13 @@
 names and call signatures the reference's model code uses
 (muxserve/flexserver/models/llama.py:35-36,75-81,200-232,257,283 for RMSNorm and
 SiluAndMul, which it imports from its vLLM fork; muxserve/flexserver/sampler.py
-for GreedySampler).  Each forwards to one entry point of libmuxattn.so; there
-is no eager fallback.
+for GreedySampler).  Each forwards to one registered operator of the package's PyTorch extension
+(libmuxtorch.so over libmuxattn.so's C ABI); there is no eager fallback.
 """
 import numpy as np
 import torch
 
-from . import ops
+from . import torch_ops as T
 
 
 class RMSNorm(torch.nn.Module):
@@ -20,14 +20,14 @@ class RMSNorm(torch.nn.Module):
         self.variance_epsilon = eps
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.rms_norm(x, self.weight.data, self.variance_epsilon)
+        return T.rms_norm(x, self.weight.data, self.variance_epsilon)
 
 
 class SiluAndMul(torch.nn.Module):
     """`forward(x)`: x [num_tokens, 2 d] -> silu(x[:, :d]) * x[:, d:]."""
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.silu_and_mul(x)
+        return T.silu_and_mul(x)
 
 
 class GreedySampler(torch.nn.Module):
@@ -56,5 +56,5 @@ class GreedySampler(torch.nn.Module):
             num_tokens = input_metadata.num_generation_tokens
         if num_tokens == 0:
             return []
-        next_tokens = ops.greedy_sample(embedding, hidden_states, self.vocab_size, num_tokens, row_index=row_index)
+        next_tokens = T.greedy_sample(embedding, hidden_states, self.vocab_size, num_tokens, row_index=row_index)
         return next_tokens.cpu().numpy().tolist()

@@ -138,16 +138,27 @@ _workspaces = {}
 
 
 def _scratch(cache: dict, nbytes: int, device, stream_ptr: int, floor: int) -> Optional[torch.Tensor]:
-    """Grow-only zero-filled scratch, one per (device, stream the launch goes
-    to).  The fill runs on torch's current stream, which need not be that
-    stream, so a new buffer is waited for once before its first use."""
+    """Grow-only zero-filled scratch, one per (device, stream the launches that
+    use it go to).  Lifetime rules, because that stream need not be torch's
+    current one (a CU-masked stream passed as ``stream=``):
+      * a new buffer is allocated and zero-filled under the device's DEFAULT
+        stream - its memory then belongs to the allocator's pool of a stream
+        that is never destroyed - and waited for once before its first use;
+      * a buffer that has become too small is only dropped after the stream it
+        is keyed to has been synchronised: launches there may still be writing
+        partial results into it, and torch would hand the block out again."""
     if nbytes == 0:
         return None
     key = (device, stream_ptr)
     ws = cache.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, floor), dtype=torch.uint8, device=device)
-        torch.cuda.current_stream(device).synchronize()
+        if ws is not None:
+            (torch.cuda.ExternalStream(stream_ptr, device=device) if stream_ptr
+             else torch.cuda.default_stream(device)).synchronize()
+        default = torch.cuda.default_stream(device)
+        with torch.cuda.stream(default):
+            ws = torch.zeros(max(nbytes, floor), dtype=torch.uint8, device=device)
+        default.synchronize()
         cache[key] = ws
     return ws
 

@@ -20,7 +20,8 @@ from ._lib import MuxLibraryMissing
 _PKG = os.path.dirname(os.path.abspath(__file__))
 TORCH_LIB_PATH = os.environ.get("MUXSERVE_TORCH_LIB", os.path.join(_PKG, "libmuxtorch.so"))
 
-OPERATORS = ("reshape_and_cache", "rope_reshape_and_cache", "rotary_neox", "paged_decode_workspace_bytes",
+OPERATORS = ("reshape_and_cache", "rope_reshape_and_cache", "multi_reshape_and_cache", "rotary_neox",
+             "paged_decode_workspace_bytes",
              "paged_decode", "multi_decode_workspace_bytes", "multi_decode", "prefill_causal", "rms_norm",
              "silu_and_mul", "greedy_sample_workspace_bytes", "greedy_sample")
 
@@ -37,3 +38,66 @@ def load():
         torch.ops.load_library(TORCH_LIB_PATH)
         _loaded = True
     return torch.ops.muxserve_amd
+
+
+
+# ---------------------------------------------------------------------------
+# The serving path's calls.  muxserve_amd.attention and muxserve_amd.layers (the
+# classes that stand in for the reference's attention layer, RMSNorm, SiluAndMul
+# and GreedySampler) reach the GPU through these: registered operators of the
+# extension, launched on torch's current stream, workspaces kept per (device,
+# stream) by muxserve_amd.ops._scratch.
+# ---------------------------------------------------------------------------
+
+def _current_stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def reshape_and_cache(k, v, k_pool, v_pool, slot_mapping, layer: int = 0, num_tokens=None) -> None:
+    load().reshape_and_cache(k, v, k_pool, v_pool, slot_mapping, int(layer), -1 if num_tokens is None else int(num_tokens))
+
+
+def rope_reshape_and_cache(positions, q, k, v, cos_sin, k_pool, v_pool, slot_mapping, layer: int = 0,
+                           num_tokens=None) -> None:
+    load().rope_reshape_and_cache(positions, q, k, v, cos_sin, k_pool, v_pool, slot_mapping, int(layer),
+                                  -1 if num_tokens is None else int(num_tokens))
+
+
+def rotary_neox(positions, q, k, cos_sin, num_tokens=None) -> None:
+    load().rotary_neox(positions, q, k, cos_sin, -1 if num_tokens is None else int(num_tokens))
+
+
+def prefill_causal(out, q, k, v, cu_seqlens, max_prompt_len: int, scale: float, num_kv_heads: int,
+                   prompt_lens=None) -> None:
+    load().prefill_causal(out, q, k, v, cu_seqlens, [] if prompt_lens is None else [int(x) for x in prompt_lens],
+                          int(max_prompt_len), float(scale), int(num_kv_heads))
+
+
+def paged_decode(out, q, k_pool, v_pool, block_tables, context_lens, max_context_len: int, scale: float,
+                 layer: int = 0, partition_size: int = 0, total_context_len: int = 0, context_lens_host=None) -> None:
+    from . import ops
+    T = load()
+    need = T.paged_decode_workspace_bytes(out, q, block_tables, context_lens, int(max_context_len), int(partition_size))
+    ws = ops._workspace(need, q.device, _current_stream_ptr(q.device))
+    if ws is None:
+        ws = torch.empty((0,), dtype=torch.uint8, device=q.device)
+    T.paged_decode(out, q, k_pool, v_pool, block_tables, context_lens, int(max_context_len), float(scale), int(layer),
+                   int(partition_size), int(total_context_len), ws, context_lens_host)
+
+
+def rms_norm(x, weight, eps: float):
+    return load().rms_norm(x, weight, float(eps))
+
+
+def silu_and_mul(x):
+    return load().silu_and_mul(x)
+
+
+def greedy_sample(embedding, hidden_states, vocab_size: int, num_rows: int, row_index=None):
+    from . import ops
+    T = load()
+    need = T.greedy_sample_workspace_bytes(int(vocab_size))
+    ws = ops._scratch(ops._sample_workspaces, need, hidden_states.device, _current_stream_ptr(hidden_states.device), 1)
+    if row_index is None:
+        row_index = torch.empty((0,), dtype=torch.int32, device=hidden_states.device)
+    return T.greedy_sample(embedding, hidden_states, int(vocab_size), int(num_rows), row_index, ws)

@@ -87,11 +87,38 @@ def test_torch_operators_equal_the_ctypes_path(dtype):
     need2 = T.multi_decode_workspace_bytes(*lists, 64)
     ws2 = torch.zeros((need2,), dtype=torch.uint8, device=DEV)
     T.multi_decode(lists[0], lists[1], k_pool, v_pool, lists[2], lists[3], lists[4], [D ** -0.5] * 2, [1, 1],
-                   [int(ctx.sum())] * 2, 64, ws2)
+                   [int(ctx.sum())] * 2, 64, ws2, [])
+    # the same with the units enumerated on the host (CPU copies of the context lengths)
+    h1, h2 = torch.zeros_like(o1), torch.zeros_like(o1)
+    host = torch.from_numpy(ctx)
+    T.multi_decode([h1, h2], lists[1], k_pool, v_pool, lists[2], lists[3], lists[4], [D ** -0.5] * 2, [1, 1],
+                   [int(ctx.sum())] * 2, 64, ws2, [host, host])
+    o4 = torch.zeros_like(o1)
+    T.paged_decode(o4, dq, k_pool, v_pool, d_bt, d_ctx, int(ctx.max()), D ** -0.5, 1, 64, 0, ws, host)
+    # the serving-path wrapper (workspace kept by the package)
+    o5 = torch.zeros_like(o1)
+    torch_ops.paged_decode(o5, dq, k_pool, v_pool, d_bt, d_ctx, int(ctx.max()), D ** -0.5, layer=1, partition_size=64,
+                           total_context_len=int(ctx.sum()), context_lens_host=host)
     o3 = torch.zeros_like(o1)
     ops.paged_decode(o3, dq2, k_pool, v_pool, d_bt, d_ctx, int(ctx.max()), D ** -0.5, layer=1, partition_size=64)
     torch.cuda.synchronize()
     assert torch.equal(_bits(f1), _bits(o1)) and torch.equal(_bits(f2), _bits(o3))
+    assert torch.equal(_bits(h1), _bits(o1)) and torch.equal(_bits(h2), _bits(o3))
+    assert torch.equal(_bits(o4), _bits(o1)) and torch.equal(_bits(o5), _bits(o1))
+    # ---- the fused cache write of two "models" against the ctypes path -----------------------
+    pa, pb = [allocate_gpu_cache(N, bs, DEV, dtype=dtype) for _ in range(2)]
+    for kp, vp in (pa, pb):
+        kp.zero_()
+        vp.zero_()
+    xa, xb = qkv.clone(), qkv.clone()
+    qa, ka, va = xa.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+    qb, kb, vb = xb.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+    ops.multi_reshape_and_cache([ops.CacheWriteCall(ka, va, slots, layer=1, positions=positions, cos_sin=cos_sin, q=qa,
+                                                    num_tokens=n)], pa[0], pa[1])
+    T.multi_reshape_and_cache([kb], [vb], pb[0], pb[1], [slots], [1], [n], [positions], [qb], [cos_sin])
+    torch.cuda.synchronize()
+    assert torch.equal(_bits(xa), _bits(xb)) and torch.equal(_bits(pa[0]), _bits(pb[0])) and \
+        torch.equal(_bits(pa[1]), _bits(pb[1]))
     # ---- stand-alone rotary, greedy sampling ---------------------------------------------
     r1 = qkv.clone().split([Hq * D, Hkv * D, Hkv * D], dim=-1)
     r2 = qkv.clone().split([Hq * D, Hkv * D, Hkv * D], dim=-1)
