@@ -61,7 +61,7 @@ def parse():
     ap.add_argument("--unfused", action="store_true", help="one launch per model instead of one fused launch")
     ap.add_argument("--workload", default="mixed3_decode",
                     choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long", "model_ops", "host_step",
-                             "cu_masks"],
+                             "cu_masks", "prefill_long"],
                     help="mixed3_decode is the headline metric; the others are the remaining synthetic "
                          "shapes, each printing its own JSON line")
     return ap.parse_args()
@@ -174,16 +174,48 @@ def bench_prefill3(args):
         for m, q, k, v, out, cu, slots, T, order in work:
             ops.reshape_and_cache(k, v, k_pool, v_pool, slots, num_tokens=T)
 
-    ms_a = _time(attn, args.steps, args.warmup)
-    ms_w = _time(write, args.steps, args.warmup)
+    ms_separate = _time(attn, args.steps, args.warmup)
+    # the three models' prompts in ONE launch, and the three cache writes in one
+    pcalls = [ops.PrefillCall(out, q, k, v, cu, [int(x) for x in m.prompt_lens], m.scale, m.num_kv_heads)
+              for m, q, k, v, out, cu, slots, T, order in work]
+    wcalls = [ops.CacheWriteCall(k, v, slots, num_tokens=T) for m, q, k, v, out, cu, slots, T, order in work]
+    ms_a = ms_separate if args.unfused else _time(lambda _: ops.multi_prefill_causal(pcalls), args.steps, args.warmup)
+    ms_w_separate = _time(write, args.steps, args.warmup)
+    ms_w = ms_w_separate if args.unfused else _time(lambda _: ops.multi_reshape_and_cache(wcalls, k_pool, v_pool),
+                                                    args.steps, args.warmup)
     tf = flops / (ms_a * 1e-3) / 1e12
     gbs = wbytes / (ms_w * 1e-3) / 1e9
     cfg = {"workload": "prefill3", "prompts_per_model": 16, "tokens": tokens, "flops": flops,
-           "cache_write_ms": ms_w, "cache_write_gbs": gbs, "cache_write_frac_of_hbm": gbs / HBM_PEAK_GBS}
+           "fused": not args.unfused, "one_launch_per_model_ms": ms_separate,
+           "cache_write_one_launch_per_model_ms": ms_w_separate, "cache_write_ms": ms_w, "cache_write_gbs": gbs, "cache_write_frac_of_hbm": gbs / HBM_PEAK_GBS}
     roof = {"bound": "mfma", "achieved": tf, "peak": 2500.0, "unit": "TFLOP/s", "frac": tf / 2500.0,
             "traffic": None, "kernel": "prefill_causal_kernel<F16>"}
     return _line("prefill causal attention tokens/s (3 models, 16 prompts each)", tokens / (ms_a * 1e-3),
                  "tokens/s", args, ms_a, cfg, roof)
+
+
+def bench_prefill_long(args):
+    """The prefill kernel alone on long prompts: 16 prompts x 2048 tokens of a
+    7B-shaped layer (32 heads x 128), fp16."""
+    import torch
+    from muxserve_amd import ops, workloads
+    from muxserve_amd.pool import HEAD_SIZE as D
+    dev, P, L, H = "cuda:0", 16, 2048, 32
+    g = torch.Generator().manual_seed(args.seed)
+    qkv = torch.randn((P * L, 3 * H * D), generator=g).half().to(dev)
+    q, k, v = qkv.split([H * D] * 3, dim=-1)
+    out = torch.empty((P * L, H * D), dtype=torch.float16, device=dev)
+    cu = torch.arange(0, P * L + 1, L, dtype=torch.int32, device=dev)
+    lens = [L] * P
+    ms = _time(lambda _: ops.prefill_causal(out, q, k, v, cu, L, D ** -0.5, H,
+                                            prompt_lens=None if args.no_prompt_lens else lens), args.steps, args.warmup)
+    flops = workloads.prefill_flops(np.asarray(lens), H)
+    tf = flops / (ms * 1e-3) / 1e12
+    cfg = {"workload": "prefill_long", "prompts": P, "prompt_len": L, "heads": H, "flops": flops}
+    roof = {"bound": "mfma", "achieved": tf, "peak": 2500.0, "unit": "TFLOP/s", "frac": tf / 2500.0,
+            "traffic": None, "kernel": "prefill_causal_kernel<F16>"}
+    return _line("prefill causal attention tokens/s (16 prompts x 2048 tokens, 32 heads)", P * L / (ms * 1e-3),
+                 "tokens/s", args, ms, cfg, roof)
 
 
 def bench_cache_write(args):
@@ -641,7 +673,7 @@ def main():
         print("bench.py: this build runs on one GPU only (no collectives or sharding); use --gpus 1",
               file=sys.stderr)
         sys.exit(2)
-    other = {"prefill3": bench_prefill3, "cache_write": bench_cache_write, "colocated": bench_colocated, "cu_masks": bench_cu_masks,
+    other = {"prefill3": bench_prefill3, "cache_write": bench_cache_write, "colocated": bench_colocated, "cu_masks": bench_cu_masks, "prefill_long": bench_prefill_long,
              "gqa_long": bench_gqa_long, "model_ops": bench_model_ops, "host_step": bench_host_step}
     if args.workload in other:
         print(json.dumps(other[args.workload](args)))

@@ -197,7 +197,7 @@ int32_t mux_paged_decode(void *out, int64_t out_row_stride, const void *q, int64
  * caller holds on the host anyway (InputMetadata.prompt_lens,
  * pipeworker.py:81-90; each <= max_prompt_len).  With them the launch holds
  * only the query tiles that exist, the heaviest of the whole batch first, and
- * prompt_order is not used; batches of more than 896 query tiles of 128 rows
+ * prompt_order is not used; batches of more than 768 query tiles of 128 rows
  * fall back to the grid sized by max_prompt_len.  The device-side cu_seqlens
  * stay authoritative for addresses and lengths (a host length shorter than the
  * device's only leaves that prompt's further query tiles unstarted).  With
@@ -209,6 +209,36 @@ int32_t mux_prefill_causal(void *out, int64_t out_row_stride,
                            const int32_t *prompt_lens_host, int32_t num_prompts,
                            int32_t max_prompt_len, int32_t num_q_heads, int32_t num_kv_heads,
                            int32_t head_size, float scale, int32_t dtype, void *stream);
+
+/* Causal prefill attention of up to MUXA_MAX_DECODE_ITEMS colocated models in
+ * ONE launch (the prompt-side counterpart of mux_multi_decode; the reference
+ * runs one attention call per model, models/llama.py:159-161): models of the
+ * same dtype whose prompts are prefilled in the same step share the grid, the
+ * heaviest query tiles of all of them first, so that the short prompts of one
+ * model fill the compute units that the long prompts of another leave idle at
+ * the end of its launch.  Field meanings are those of mux_prefill_causal.  The
+ * shared grid needs prompt_lens_host for every item and at most 768 query tiles
+ * of 128 rows in all; otherwise the call falls back to one launch per model.
+ * Results are bit-identical to the per-model calls.  `items` is a HOST array. */
+typedef struct MuxPrefillItem {
+  void *out;
+  int64_t out_row_stride;
+  const void *q;
+  int64_t q_row_stride;
+  const void *k;
+  const void *v;
+  int64_t kv_row_stride;
+  const int32_t *cu_seqlens;         /* DEVICE int32 [num_prompts + 1] */
+  const int32_t *prompt_lens_host;   /* HOST int32 [num_prompts] */
+  int32_t num_prompts;
+  int32_t max_prompt_len;
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  float scale;
+} MuxPrefillItem;
+
+int32_t mux_multi_prefill_causal(const MuxPrefillItem *items, int32_t n_items, int32_t head_size,
+                                 int32_t dtype, void *stream);
 
 /* ---- Rotary position embedding --------------------------------------------
  * The attention layer of the reference is PagedAttentionWithRoPE constructed

@@ -117,6 +117,16 @@ class MuxDecodeItem(ctypes.Structure):
     ]
 
 
+class MuxPrefillItem(ctypes.Structure):
+    _fields_ = [
+        ("out", c_vp), ("out_row_stride", c_i64), ("q", c_vp), ("q_row_stride", c_i64),
+        ("k", c_vp), ("v", c_vp), ("kv_row_stride", c_i64),
+        ("cu_seqlens", c_vp), ("prompt_lens_host", c_vp),
+        ("num_prompts", c_i32), ("max_prompt_len", c_i32), ("num_q_heads", c_i32), ("num_kv_heads", c_i32),
+        ("scale", c_f32),
+    ]
+
+
 class MuxCacheWriteItem(ctypes.Structure):
     _fields_ = [
         ("positions", c_vp), ("q", c_vp), ("q_row_stride", c_i64),
@@ -132,6 +142,7 @@ ATTN_SIGNATURES = {
     "mux_last_hip_error": (c_i32, []),
     "mux_reshape_and_cache": (c_i32, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i32, c_i32,
                                       c_i32, c_i32, c_i32, c_i32, c_i32, c_vp]),
+    "mux_multi_prefill_causal": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_vp]),
     "mux_multi_rope_reshape_and_cache": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_vp]),
     "mux_paged_decode_workspace_bytes": (c_sz, [c_vp, c_i32, c_i32]),
     "mux_paged_decode_workspace_init": (c_i32, [c_vp, c_sz, c_vp]),

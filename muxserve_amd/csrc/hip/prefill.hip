@@ -23,6 +23,9 @@
 // The next tile's global loads are issued before the current tile's math.
 #include "mux_common.h"
 
+#include <algorithm>
+#include <vector>
+
 namespace mux {
 
 typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
@@ -36,7 +39,7 @@ constexpr int kBN = 32;                  // keys per tile
 constexpr int kNKB = kBN / 32;           // 32-key blocks (one MFMA row block) per tile
 
 // Query tiles listed in the kernel argument (its size limit is 4 KiB).
-constexpr int kMaxPairs = 896;
+constexpr int kMaxPairs = 768;
 
 union Frag {
   u32x4 u;
@@ -67,24 +70,36 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   }
 }
 
-struct PrefillParams {
+// One model's prompts (several colocated models can share a launch).
+struct PrefillItemDev {
   uint16_t *out;
   const uint16_t *q, *k, *v;
   int64_t out_stride, q_stride, kv_stride;
   const int32_t *cu_seqlens;
-  const int32_t *prompt_order;   // optional: prompts in the order their workgroups should start
   int32_t ratio;          // query heads per kv head
-  int32_t q_tiles;        // 128-row query tiles per prompt (of the longest prompt)
   int32_t num_kv_heads;
-  int32_t num_groups;     // (prompt, kv head) pairs
+  int32_t num_prompts;
+  int32_t kv_per_xcd;     // ceil(num_kv_heads / 8)
   float scale_log2;
   int32_t out_rows_16b;   // out and its row stride allow 16-byte stores
+};
+
+struct PrefillParams {
+  PrefillItemDev it[MUXA_MAX_DECODE_ITEMS];
+  const int32_t *prompt_order;   // dense grid, optional: prompts in the order their workgroups should start
+  int32_t q_tiles;        // dense grid: 128-row query tiles per prompt (of the longest prompt)
+  int32_t num_groups;     // dense grid: (prompt, kv head) pairs
   // Compact grid (the caller gave the prompt lengths on the host): the query
-  // tiles that exist, heaviest first, as prompt << 16 | tile; 0 pairs = dense grid.
+  // tiles that exist, the heaviest of all models first, as
+  // model << 28 | prompt << 12 | tile; every pair takes slots_per_pair workgroups
+  // on each XCD (the largest model's kv heads per XCD x query heads per kv head;
+  // the surplus of smaller models leaves at once).  0 pairs = dense grid, one model.
   int32_t n_pairs;
-  int32_t kv_per_xcd;     // ceil(num_kv_heads / 8)
+  int32_t slots_per_pair;
   uint32_t pairs[kMaxPairs];
 };
+static_assert(sizeof(PrefillParams) <= 4096, "kernel argument segment");
+constexpr int kPairTileBits = 12;       // tile in bits 0-11, prompt in bits 12-27, model in bits 28-30
 
 // K and V tiles go from global memory straight into LDS
 // (global_load_lds_dwordx4: lane l's 16 bytes land at base + 16 l), row-major
@@ -101,6 +116,18 @@ typedef short v4i16 __attribute__((ext_vector_type(4)));
 #define MUX_PF_PRIO_MFMA 1
 #define MUX_PF_PRIO_VALU 0
 constexpr int kTileElems = kBN * kHeadSize;          // one unpadded row-major tile
+// The swizzle: the 16-byte chunk c of tile row r sits at chunk position
+// c ^ swz(r), swz(r) = the low three bits of r rotated left by one, bit 3 kept.
+// LDS has 32 banks of 4 bytes: a 256-byte row covers them twice, so only the low
+// three bits of a chunk position choose the banks.  The K fragments are read 8
+// rows at a time (one chunk each, ds_read_b128): the rotated low bits of 8
+// consecutive rows are all different.  The V^T fragments are read 16 lanes at a
+// time (ds_read_b64_tr_b16) over 4 consecutive rows x 2 neighbouring chunks x
+// the two halves of a chunk: the rows' two low bits land in position bits 1-2
+// and the chunk pair in bit 0 - again all different.  (With the plain c ^ r the
+// four rows and the chunk pair shared two position bits: a two-way conflict on
+// every V^T read.)
+__device__ __forceinline__ int swz(int row) { return ((row & 3) << 1) | ((row >> 2) & 1) | (row & 8); }
 
 template <typename T>
 __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillParams P) {
@@ -118,39 +145,43 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
   // heads of one (prompt, kv head) pair - are therefore given ids that are equal
   // mod 8.
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int num_prompts = P.num_groups / P.num_kv_heads;
-  int prompt, hk, hq, q0;
+  int item = 0, prompt, hk, hq, q0, rem = 0;
+  uint32_t pair = 0;
   if (P.n_pairs > 0) {
-    // Compact grid: only query tiles that exist, the heaviest of the whole batch
-    // first; kv head hk of prompt p lives on XCD (hk + p) % 8 (rotated by the
-    // prompt so that head counts that are no multiple of 8 load the XCDs evenly).
-    const int per_pair = P.kv_per_xcd * P.ratio;
-    const int pi = slot / per_pair;
+    // Compact grid: only query tiles that exist, the heaviest of the whole launch first.
+    const int pi = slot / P.slots_per_pair;
     if (pi >= P.n_pairs) return;
-    const int rem = slot - pi * per_pair;
-    const uint32_t pair = P.pairs[pi];
+    rem = slot - pi * P.slots_per_pair;
+    pair = P.pairs[pi];
+    item = min(static_cast<int>(pair >> 28), MUXA_MAX_DECODE_ITEMS - 1);
+  }
+  const PrefillItemDev I = P.it[item];
+  if (P.n_pairs > 0) {
+    // kv head hk of prompt p lives on XCD (hk + p) % 8 (rotated by the prompt so
+    // that head counts that are no multiple of 8 load the XCDs evenly).
+    if (rem >= I.kv_per_xcd * I.ratio) return;
     // (clamped: a malformed list costs results, never a stray read)
-    prompt = min(static_cast<int>(pair >> 16), num_prompts - 1);
-    q0 = static_cast<int>(pair & 0xffffu) * kBM;
-    hk = ((xcd - prompt) & 7) + 8 * (rem / P.ratio);
-    if (hk >= P.num_kv_heads) return;
-    hq = hk * P.ratio + rem % P.ratio;
+    prompt = min(static_cast<int>((pair >> kPairTileBits) & 0xffffu), I.num_prompts - 1);
+    q0 = static_cast<int>(pair & ((1u << kPairTileBits) - 1)) * kBM;
+    hk = ((xcd - prompt) & 7) + 8 * (rem / I.ratio);
+    if (hk >= I.num_kv_heads) return;
+    hq = hk * I.ratio + rem % I.ratio;
   } else {
     // Dense grid: every prompt gets the tiles of the longest one, heaviest first;
     // (prompt, kv head) groups go round-robin over the XCDs.
-    const int per_group = P.ratio * P.q_tiles;
+    const int per_group = I.ratio * P.q_tiles;
     const int group = (slot / per_group) * 8 + xcd;
     if (group >= P.num_groups) return;
     const int in_group = slot % per_group;
-    const int prompt_rank = group / P.num_kv_heads;
+    const int prompt_rank = group / I.num_kv_heads;
     // (an entry outside the batch is clamped, as above)
-    prompt = P.prompt_order ? min(max(P.prompt_order[prompt_rank], 0), num_prompts - 1) : prompt_rank;
-    hk = group % P.num_kv_heads;
-    hq = hk * P.ratio + in_group / P.q_tiles;
+    prompt = P.prompt_order ? min(max(P.prompt_order[prompt_rank], 0), I.num_prompts - 1) : prompt_rank;
+    hk = group % I.num_kv_heads;
+    hq = hk * I.ratio + in_group / P.q_tiles;
     q0 = (P.q_tiles - 1 - in_group % P.q_tiles) * kBM;
   }
-  const int seq_begin = P.cu_seqlens[prompt];
-  const int len = P.cu_seqlens[prompt + 1] - seq_begin;
+  const int seq_begin = I.cu_seqlens[prompt];
+  const int len = I.cu_seqlens[prompt + 1] - seq_begin;
   if (q0 >= len) return;
 
   const int qcol = lane & 31;            // this lane's query column / fragment row
@@ -162,7 +193,7 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
   Frag qf[8];
   {
     const bool ok = my_q < len;
-    const uint16_t *qp = P.q + static_cast<int64_t>(seq_begin + (ok ? my_q : 0)) * P.q_stride + hq * D + 8 * half;
+    const uint16_t *qp = I.q + static_cast<int64_t>(seq_begin + (ok ? my_q : 0)) * I.q_stride + hq * D + 8 * half;
 #pragma unroll
     for (int s = 0; s < 8; ++s) qf[s].u = ok ? *reinterpret_cast<const u32x4 *>(qp + 16 * s) : u32x4{0, 0, 0, 0};
   }
@@ -179,9 +210,9 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
   const int n_tiles = (kv_end + kBN - 1) / kBN;
 
   // ---- tile staging -------------------------------------------------------------------
-  const uint32_t row_bytes = static_cast<uint32_t>(P.kv_stride) * 2u;
-  const char *kbase = reinterpret_cast<const char *>(P.k + static_cast<int64_t>(seq_begin) * P.kv_stride + hk * D);
-  const char *vbase = reinterpret_cast<const char *>(P.v + static_cast<int64_t>(seq_begin) * P.kv_stride + hk * D);
+  const uint32_t row_bytes = static_cast<uint32_t>(I.kv_stride) * 2u;
+  const char *kbase = reinterpret_cast<const char *>(I.k + static_cast<int64_t>(seq_begin) * I.kv_stride + hk * D);
+  const char *vbase = reinterpret_cast<const char *>(I.v + static_cast<int64_t>(seq_begin) * I.kv_stride + hk * D);
   const uint32_t tile_bytes = kBN * row_bytes;
   const uint32_t last_row = static_cast<uint32_t>(len - 1) * row_bytes;
   // Rows past the prompt re-read its last row: finite data whose probability is
@@ -189,11 +220,11 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
 
   // Instruction i of wave w fills KiB 4 i + w of a tile = rows 16 i + 4 w .. +3;
   // lane l sits at row 16 i + 4 w + l/16, position l%16, and fetches chunk
-  // position ^ (row % 16) - the same chunk for every i.
+  // position ^ swz(row) - the same chunk for every i (rows 16 apart swizzle alike).
   constexpr int kLoads = kBN / 16;         // such instructions per wave, tile and operand
   uint32_t koff[kLoads];
   const int row0 = 4 * wave + (lane >> 4);
-  const int chunk0 = (lane & 15) ^ (row0 & 15);
+  const int chunk0 = (lane & 15) ^ swz(row0);
 #pragma unroll
   for (int i = 0; i < kLoads; ++i) koff[i] = static_cast<uint32_t>(row0 + 16 * i) * row_bytes + 16u * chunk0;
   const uint32_t kmax = last_row + 16u * chunk0;
@@ -217,8 +248,9 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
   {
     const int jrow = (lane & 15) >> 2, m = lane & 3;
     const int rl = 4 * half + jrow, cl = 2 * ((lane >> 4) & 1) + (m >> 1);
-    v_lane_base[0] = rl * D + 8 * (cl ^ rl) + 4 * (m & 1);
-    v_lane_base[1] = rl * D + 8 * (cl ^ rl ^ 4) + 4 * (m & 1);
+    // rl < 8, cl < 4: the lane's part of the position is cl ^ swz(rl), below 8.
+    v_lane_base[0] = rl * D + 8 * (cl ^ swz(rl)) + 4 * (m & 1);
+    v_lane_base[1] = rl * D + 8 * (cl ^ swz(rl) ^ 4) + 4 * (m & 1);
   }
   dma_tile(0);
   for (int t = 0; t < n_tiles; ++t) {
@@ -251,7 +283,7 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
       auto read_k = [&](int j) {
         Frag f;
         const int row = 32 * (j % kNKB) + qcol, chunk = 2 * (j / kNKB) + half;
-        f.u = *reinterpret_cast<const u32x4 *>(Kt + row * D + 8 * (chunk ^ (row & 15)));
+        f.u = *reinterpret_cast<const u32x4 *>(Kt + row * D + 8 * (chunk ^ swz(row)));
         return f;
       };
       Frag ring[kDepth];
@@ -290,7 +322,7 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
     const float m_new = fmaxf(m_run, mx);
     // Rows past the prompt may have no valid key at all; keep them finite.
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float neg_m = -m_use * P.scale_log2;
+    const float neg_m = -m_use * I.scale_log2;
     float psum = 0.f;
     Frag pf[2 * kNKB];                          // B fragments: [kb][step] -> index 2 kb + st
     // bf16 keeps only 8 mantissa bits of a probability, which alone would cost
@@ -301,7 +333,7 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
     for (int kb = 0; kb < kNKB; ++kb) {
       float p[16];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) p[i] = fast_exp2(__builtin_fmaf(sacc[kb][i], P.scale_log2, neg_m));
+      for (int i = 0; i < 16; ++i) p[i] = fast_exp2(__builtin_fmaf(sacc[kb][i], I.scale_log2, neg_m));
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
         uint32_t w[4];
@@ -326,7 +358,7 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
     // The running max rises only in the first tiles of a row; skip the rescale
     // of the 64 accumulators when no lane of the wave needs it.
     if (__builtin_amdgcn_ballot_w64(m_use > m_run) != 0) {
-      const float alpha = fast_exp2((m_run - m_use) * P.scale_log2);
+      const float alpha = fast_exp2((m_run - m_use) * I.scale_log2);
       l_run *= alpha;
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb)
@@ -347,7 +379,7 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
         // group receives dim i of rows 0..3.  Here a group covers dims
         // 32 mb + 16 (lane/16 % 2) .. +15 and keys 16 ks + 4 half (+ 8) .. +3.
         // Address: row = 16 ks + 8 hsel + rl with rl = 4 half + jrow, chunk =
-        // 4 mb + cl, position = chunk ^ (row % 16) = (cl ^ rl) ^ 4 (mb ^ 2 hsel).
+        // 4 mb + cl, position = chunk ^ swz(row) = (cl ^ swz(rl)) ^ 4 (mb ^ 2 hsel).
         // The lane part cl ^ rl is below 8, so bit 3 of the constant part adds
         // and only its bit 2 (mb odd) has to be folded into the lane's base:
         // two bases per lane, everything else is an immediate offset.
@@ -383,7 +415,7 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
   // ---- normalise and store: register i of block mb is d = 32 mb + 8 (i/4) + 4 half + i%4 ------
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = 1.f / l_tot;
-  if (P.out_rows_16b) {
+  if (I.out_rows_16b) {
     // Through LDS, so that the rows go out as whole 256-byte runs (16 bytes per
     // lane, four rows per instruction) instead of 8-byte pieces of 32 rows: the
     // tile buffers are free once every wave has left the loop.
@@ -407,12 +439,12 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
       const int r = 4 * it + (lane >> 4);
       if (wq0 + r < len) {
         const u32x4 x = *reinterpret_cast<const u32x4 *>(&stage[r * kORow + 8 * chunk]);
-        *reinterpret_cast<u32x4 *>(P.out + static_cast<int64_t>(seq_begin + wq0 + r) * P.out_stride + hq * D +
+        *reinterpret_cast<u32x4 *>(I.out + static_cast<int64_t>(seq_begin + wq0 + r) * I.out_stride + hq * D +
                                    8 * chunk) = x;
       }
     }
   } else if (my_q < len) {
-    uint16_t *op = P.out + static_cast<int64_t>(seq_begin + my_q) * P.out_stride + hq * D + 4 * half;
+    uint16_t *op = I.out + static_cast<int64_t>(seq_begin + my_q) * I.out_stride + hq * D + 4 * half;
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
@@ -426,6 +458,160 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
 
 }  // namespace mux
 
+namespace mux {
+namespace {
+
+int32_t check_prefill_item(const MuxPrefillItem &it, int32_t head_size) {
+  // (pointers are only required when there is something to do)
+  const bool work = it.num_prompts > 0 && it.max_prompt_len > 0;
+  if (work && (!it.out || !it.q || !it.k || !it.v || !it.cu_seqlens)) return MUXA_EINVAL;
+  if (it.num_prompts < 0 || it.max_prompt_len < 0 || it.num_q_heads <= 0 || it.num_kv_heads <= 0) return MUXA_EINVAL;
+  if (it.num_q_heads % it.num_kv_heads != 0) return MUXA_EINVAL;
+  if (head_size != kHeadSize) return MUXA_EUNSUPPORTED;
+  if (it.q_row_stride < static_cast<int64_t>(it.num_q_heads) * kHeadSize ||
+      it.out_row_stride < static_cast<int64_t>(it.num_q_heads) * kHeadSize ||
+      it.kv_row_stride < static_cast<int64_t>(it.num_kv_heads) * kHeadSize)
+    return MUXA_EINVAL;
+  // 16-byte fragment loads and 8-byte output stores.
+  if (it.q_row_stride % 8 || it.kv_row_stride % 8 || it.out_row_stride % 4) return MUXA_EINVAL;
+  const uintptr_t a16 =
+      reinterpret_cast<uintptr_t>(it.q) | reinterpret_cast<uintptr_t>(it.k) | reinterpret_cast<uintptr_t>(it.v);
+  if ((a16 & 15u) || (reinterpret_cast<uintptr_t>(it.out) & 7u)) return MUXA_EINVAL;
+  // K/V rows of one prompt are addressed with 32-bit byte offsets.
+  if (static_cast<int64_t>(it.max_prompt_len + kBM + 2 * kBN) * it.kv_row_stride * 2 >= (int64_t{1} << 32))
+    return MUXA_EUNSUPPORTED;
+  if (it.prompt_lens_host != nullptr)
+    for (int p = 0; p < it.num_prompts; ++p)
+      if (it.prompt_lens_host[p] < 0 || it.prompt_lens_host[p] > it.max_prompt_len) return MUXA_EINVAL;
+  return MUXA_OK;
+}
+
+PrefillItemDev device_item(const MuxPrefillItem &it) {
+  PrefillItemDev d;
+  d.out = static_cast<uint16_t *>(it.out);
+  d.q = static_cast<const uint16_t *>(it.q);
+  d.k = static_cast<const uint16_t *>(it.k);
+  d.v = static_cast<const uint16_t *>(it.v);
+  d.out_stride = it.out_row_stride;
+  d.q_stride = it.q_row_stride;
+  d.kv_stride = it.kv_row_stride;
+  d.cu_seqlens = it.cu_seqlens;
+  d.ratio = it.num_q_heads / it.num_kv_heads;
+  d.num_kv_heads = it.num_kv_heads;
+  d.num_prompts = it.num_prompts;
+  d.kv_per_xcd = (it.num_kv_heads + 7) / 8;
+  d.scale_log2 = it.scale * 1.4426950408889634f;
+  d.out_rows_16b = (reinterpret_cast<uintptr_t>(it.out) & 15u) == 0 && it.out_row_stride % 8 == 0;
+  return d;
+}
+
+hipError_t launch_prefill(const PrefillParams &P, int64_t n_wg, int32_t dtype, hipStream_t st) {
+  const dim3 grid(static_cast<uint32_t>(n_wg));
+  if (dtype == MUXA_DTYPE_F16) hipLaunchKernelGGL((prefill_causal_kernel<F16>), grid, dim3(256), 0, st, P);
+  else hipLaunchKernelGGL((prefill_causal_kernel<BF16>), grid, dim3(256), 0, st, P);
+  return hipGetLastError();
+}
+
+// One model on the grid sized by its longest prompt (no host-side lengths, or too
+// many query tiles for the kernel argument).
+int32_t launch_dense(const MuxPrefillItem &it, const int32_t *prompt_order, int32_t dtype, hipStream_t st) {
+  PrefillParams P = {};
+  P.it[0] = device_item(it);
+  P.prompt_order = prompt_order;
+  P.q_tiles = (it.max_prompt_len + kBM - 1) / kBM;
+  P.num_groups = it.num_prompts * it.num_kv_heads;
+  const int64_t n_wg = static_cast<int64_t>((P.num_groups + 7) / 8) * 8 * P.it[0].ratio * P.q_tiles;
+  if (n_wg > 0x7fffffff || P.q_tiles > 0xffff) return MUXA_EUNSUPPORTED;
+  hipError_t e = launch_prefill(P, n_wg, dtype, st);
+  if (e != hipSuccess) return hip_fail(e);
+  return MUXA_OK;
+}
+
+// items[first .. first + n): one launch over the query tiles that exist, the
+// heaviest (most keys) of all models first; false when they do not fit the
+// kernel argument.
+bool launch_compact(const MuxPrefillItem *items, int n, int32_t dtype, hipStream_t st, int32_t *rc) {
+  PrefillParams P = {};
+  int64_t total = 0;
+  int max_tiles = 0, slots = 0, n_dev = 0;
+  int dev_of[MUXA_MAX_DECODE_ITEMS];
+  for (int i = 0; i < n; ++i) {
+    const MuxPrefillItem &it = items[i];
+    dev_of[i] = -1;
+    if (it.num_prompts == 0 || it.max_prompt_len == 0) continue;
+    if (it.prompt_lens_host == nullptr || it.num_prompts > 0xffff) return false;
+    int64_t tiles = 0;
+    for (int p = 0; p < it.num_prompts; ++p) tiles += (it.prompt_lens_host[p] + kBM - 1) / kBM;
+    if (tiles == 0) continue;
+    total += tiles;
+    max_tiles = std::max(max_tiles, (it.max_prompt_len + kBM - 1) / kBM);
+    dev_of[i] = n_dev;
+    P.it[n_dev] = device_item(it);
+    slots = std::max(slots, P.it[n_dev].kv_per_xcd * P.it[n_dev].ratio);
+    ++n_dev;
+  }
+  *rc = MUXA_OK;
+  if (total == 0) return true;
+  if (total > kMaxPairs || max_tiles > (1 << kPairTileBits)) return false;
+  // Order: prompt by prompt, the longest prompt of all models first, and within a
+  // prompt the heaviest query tile (most keys) first.  The query tiles and query
+  // heads that read the same K/V then run at the same time on one XCD and walk
+  // the keys from the start together, so a K/V tile is fetched from memory once
+  // and found in that XCD's L2 by the others (tile by tile over the whole batch
+  // instead - every stream of the batch live at once - the 16 x 2048-token shape
+  // re-read K/V from memory at 4.6 TB/s and ran 1.2 x slower), and the launch
+  // ends with the short prompts' small tiles.
+  struct Group {
+    int item, prompt, len;
+  };
+  std::vector<Group> groups;
+  for (int i = 0; i < n; ++i) {
+    if (dev_of[i] < 0) continue;
+    for (int p = 0; p < items[i].num_prompts; ++p)
+      if (items[i].prompt_lens_host[p] > 0) groups.push_back({i, p, items[i].prompt_lens_host[p]});
+  }
+  std::stable_sort(groups.begin(), groups.end(), [](const Group &a, const Group &b) { return a.len > b.len; });
+  int np = 0;
+  for (const Group &g : groups)
+    for (int t = (g.len + kBM - 1) / kBM - 1; t >= 0; --t)
+      P.pairs[np++] = (static_cast<uint32_t>(dev_of[g.item]) << 28) |
+                      (static_cast<uint32_t>(g.prompt) << kPairTileBits) | static_cast<uint32_t>(t);
+  P.n_pairs = np;
+  P.slots_per_pair = slots;
+  const int64_t n_wg = static_cast<int64_t>(np) * slots * 8;
+  if (n_wg > 0x7fffffff) {
+    *rc = MUXA_EUNSUPPORTED;
+    return true;
+  }
+  hipError_t e = launch_prefill(P, n_wg, dtype, st);
+  if (e != hipSuccess) *rc = hip_fail(e);
+  return true;
+}
+
+}  // namespace
+}  // namespace mux
+
+extern "C" int32_t mux_multi_prefill_causal(const MuxPrefillItem *items, int32_t n_items, int32_t head_size,
+                                            int32_t dtype, void *stream) {
+  using namespace mux;
+  if (!items || n_items <= 0 || n_items > MUXA_MAX_DECODE_ITEMS) return MUXA_EINVAL;
+  if (dtype != MUXA_DTYPE_F16 && dtype != MUXA_DTYPE_BF16) return MUXA_EUNSUPPORTED;
+  for (int i = 0; i < n_items; ++i) {
+    const int32_t rc = check_prefill_item(items[i], head_size);
+    if (rc != MUXA_OK) return rc;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  int32_t rc = MUXA_OK;
+  if (launch_compact(items, n_items, dtype, st, &rc)) return rc;
+  // Not all in one kernel argument: one launch per model, compact where possible.
+  for (int i = 0; i < n_items; ++i) {
+    if (items[i].num_prompts == 0 || items[i].max_prompt_len == 0) continue;
+    if (!launch_compact(items + i, 1, dtype, st, &rc)) rc = launch_dense(items[i], nullptr, dtype, st);
+    if (rc != MUXA_OK) return rc;
+  }
+  return MUXA_OK;
+}
+
 extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const void *q, int64_t q_row_stride,
                                       const void *k, const void *v, int64_t kv_row_stride,
                                       const int32_t *cu_seqlens, const int32_t *prompt_order,
@@ -433,67 +619,27 @@ extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const v
                                       int32_t max_prompt_len, int32_t num_q_heads, int32_t num_kv_heads,
                                       int32_t head_size, float scale, int32_t dtype, void *stream) {
   using namespace mux;
-  // (pointers are only required when there is something to do)
-  const bool work = num_prompts > 0 && max_prompt_len > 0;
-  if (work && (!out || !q || !k || !v || !cu_seqlens)) return MUXA_EINVAL;
-  if (num_prompts < 0 || max_prompt_len < 0 || num_q_heads <= 0 || num_kv_heads <= 0) return MUXA_EINVAL;
-  if (num_q_heads % num_kv_heads != 0) return MUXA_EINVAL;
-  if (head_size != kHeadSize) return MUXA_EUNSUPPORTED;
   if (dtype != MUXA_DTYPE_F16 && dtype != MUXA_DTYPE_BF16) return MUXA_EUNSUPPORTED;
-  if (q_row_stride < static_cast<int64_t>(num_q_heads) * kHeadSize ||
-      out_row_stride < static_cast<int64_t>(num_q_heads) * kHeadSize ||
-      kv_row_stride < static_cast<int64_t>(num_kv_heads) * kHeadSize)
-    return MUXA_EINVAL;
-  // 16-byte fragment loads and 8-byte output stores.
-  if (q_row_stride % 8 || kv_row_stride % 8 || out_row_stride % 4) return MUXA_EINVAL;
-  const uintptr_t a16 = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v);
-  if ((a16 & 15u) || (reinterpret_cast<uintptr_t>(out) & 7u)) return MUXA_EINVAL;
-  // K/V rows of one prompt are addressed with 32-bit byte offsets.
-  if (static_cast<int64_t>(max_prompt_len + kBM + 2 * kBN) * kv_row_stride * 2 >= (int64_t{1} << 32)) return MUXA_EUNSUPPORTED;
+  MuxPrefillItem it = {};
+  it.out = out;
+  it.out_row_stride = out_row_stride;
+  it.q = q;
+  it.q_row_stride = q_row_stride;
+  it.k = k;
+  it.v = v;
+  it.kv_row_stride = kv_row_stride;
+  it.cu_seqlens = cu_seqlens;
+  it.prompt_lens_host = prompt_lens_host;
+  it.num_prompts = num_prompts;
+  it.max_prompt_len = max_prompt_len;
+  it.num_q_heads = num_q_heads;
+  it.num_kv_heads = num_kv_heads;
+  it.scale = scale;
+  const int32_t rc0 = check_prefill_item(it, head_size);
+  if (rc0 != MUXA_OK) return rc0;
   if (num_prompts == 0 || max_prompt_len == 0) return MUXA_OK;
-
-  PrefillParams P;
-  P.out = static_cast<uint16_t *>(out);
-  P.q = static_cast<const uint16_t *>(q);
-  P.k = static_cast<const uint16_t *>(k);
-  P.v = static_cast<const uint16_t *>(v);
-  P.out_stride = out_row_stride;
-  P.q_stride = q_row_stride;
-  P.kv_stride = kv_row_stride;
-  P.cu_seqlens = cu_seqlens;
-  P.prompt_order = prompt_order;
-  P.ratio = num_q_heads / num_kv_heads;
-  P.q_tiles = (max_prompt_len + kBM - 1) / kBM;
-  P.num_kv_heads = num_kv_heads;
-  P.num_groups = num_prompts * num_kv_heads;
-  P.scale_log2 = scale * 1.4426950408889634f;
-  P.out_rows_16b = (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && out_row_stride % 8 == 0;
-  int64_t n_wg = static_cast<int64_t>((P.num_groups + 7) / 8) * 8 * P.ratio * P.q_tiles;
-  P.n_pairs = 0;
-  P.kv_per_xcd = (num_kv_heads + 7) / 8;
-  if (prompt_lens_host != nullptr && num_prompts <= 0xffff) {
-    // The query tiles that exist, heaviest (most keys) first; ties: as packed.
-    int64_t total = 0;
-    for (int p = 0; p < num_prompts; ++p) {
-      if (prompt_lens_host[p] < 0 || prompt_lens_host[p] > max_prompt_len) return MUXA_EINVAL;
-      total += (prompt_lens_host[p] + kBM - 1) / kBM;
-    }
-    if (total == 0) return MUXA_OK;
-    if (total <= kMaxPairs) {
-      int n = 0;
-      for (int t = P.q_tiles - 1; t >= 0; --t)
-        for (int p = 0; p < num_prompts; ++p)
-          if (t * kBM < prompt_lens_host[p]) P.pairs[n++] = (static_cast<uint32_t>(p) << 16) | static_cast<uint32_t>(t);
-      P.n_pairs = n;
-      n_wg = static_cast<int64_t>(n) * P.kv_per_xcd * P.ratio * 8;
-    }
-  }
-  if (n_wg > 0x7fffffff || P.q_tiles > 0xffff) return MUXA_EUNSUPPORTED;
-  const dim3 grid(static_cast<uint32_t>(n_wg));
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (dtype == MUXA_DTYPE_F16) hipLaunchKernelGGL((prefill_causal_kernel<F16>), grid, dim3(256), 0, st, P);
-  else hipLaunchKernelGGL((prefill_causal_kernel<BF16>), grid, dim3(256), 0, st, P);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return hip_fail(e);
-  return MUXA_OK;
+  int32_t rc = MUXA_OK;
+  if (launch_compact(&it, 1, dtype, st, &rc)) return rc;
+  return launch_dense(it, prompt_order, dtype, st);
 }

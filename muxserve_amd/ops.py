@@ -256,6 +256,54 @@ def prefill_causal(out, q, k, v, cu_seqlens: torch.Tensor, max_prompt_len: int, 
     _lib.check_attn(rc, "mux_prefill_causal")
 
 
+@dataclass
+class PrefillCall:
+    """One model's prompts of a prefill step (an element of a fused launch)."""
+    out: torch.Tensor             # [>=T, Hq*128]
+    q: torch.Tensor               # [>=T, Hq*128]
+    k: torch.Tensor               # [>=T, Hkv*128]
+    v: torch.Tensor
+    cu_seqlens: torch.Tensor      # int32 [P+1], device
+    prompt_lens: List[int]        # host-side lengths
+    scale: float
+    num_kv_heads: int
+
+    def to_item(self) -> _lib.MuxPrefillItem:
+        out, q, k, v, cu = self.out, self.q, self.k, self.v, self.cu_seqlens
+        _need_cuda(out, q, k, v, cu)
+        if cu.dtype != torch.int32 or cu.dim() != 1 or not cu.is_contiguous() or cu.shape[0] != len(self.prompt_lens) + 1:
+            raise ValueError("cu_seqlens: expected contiguous int32 [P+1] for P host-side prompt lengths")
+        if q.shape[1] % HEAD_SIZE or k.shape[1] != self.num_kv_heads * HEAD_SIZE or k.shape != v.shape:
+            raise ValueError("q [T, Hq*128], k/v [T, Hkv*128] expected")
+        if not (q.dtype == k.dtype == v.dtype == out.dtype):
+            raise TypeError("q, k, v, out dtypes differ")
+        kv_stride = _rows(k, "k")
+        if _rows(v, "v") != kv_stride:
+            raise ValueError("k and v row strides differ")
+        self._lens = (ctypes.c_int32 * len(self.prompt_lens))(*[int(x) for x in self.prompt_lens])   # kept alive by self
+        it = _lib.MuxPrefillItem()
+        it.out, it.out_row_stride, it.q, it.q_row_stride = out.data_ptr(), _rows(out, "out"), q.data_ptr(), _rows(q, "q")
+        it.k, it.v, it.kv_row_stride = k.data_ptr(), v.data_ptr(), kv_stride
+        it.cu_seqlens, it.prompt_lens_host = cu.data_ptr(), ctypes.addressof(self._lens)
+        it.num_prompts, it.max_prompt_len = len(self.prompt_lens), max([int(x) for x in self.prompt_lens], default=0)
+        it.num_q_heads, it.num_kv_heads, it.scale = q.shape[1] // HEAD_SIZE, int(self.num_kv_heads), float(self.scale)
+        return it
+
+
+def multi_prefill_causal(calls: List[PrefillCall], stream=None) -> None:
+    """Causal prefill attention of several colocated models' prompts in one launch
+    (the heaviest query tiles of all models first); bit-identical to one
+    prefill_causal call per model."""
+    if not 1 <= len(calls) <= _lib.MUXA_MAX_DECODE_ITEMS:
+        raise ValueError(f"1..{_lib.MUXA_MAX_DECODE_ITEMS} models per launch")
+    if len({c.q.dtype for c in calls}) != 1:
+        raise TypeError("the models of a fused launch must share a dtype")
+    items = (_lib.MuxPrefillItem * len(calls))(*[c.to_item() for c in calls])
+    rc = _lib.attn().mux_multi_prefill_causal(ctypes.addressof(items), len(calls), HEAD_SIZE, _dtype_code(calls[0].q),
+                                              _stream_ptr(stream))
+    _lib.check_attn(rc, "mux_multi_prefill_causal")
+
+
 def rotary_neox(positions: torch.Tensor, q: torch.Tensor, k: torch.Tensor, cos_sin: torch.Tensor,
                 num_tokens: Optional[int] = None, stream=None) -> None:
     """NeoX rotary embedding in place on q [T_pad, Hq*128] and k [T_pad, Hkv*128];

@@ -237,6 +237,79 @@ def test_config3_prefill_then_cache_write_bit_exact():
     assert torch.equal(dv_pool.cpu().view(torch.int16), hv_pool.view(torch.int16))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_prefill_of_three_models_equals_one_launch_per_model(dtype):
+    """mux_multi_prefill_causal over config 3's three shapes (plus a grouped-query
+    model and a model without prompts) against one mux_prefill_causal per model:
+    every output bitwise equal - the shared grid only changes which workgroup
+    runs when - and the fused cache write of the same step bitwise equal to the
+    oracle's scatter."""
+    _announce(f"fused prefill, three models {dtype}")
+    bs = 16
+    models = workloads.config3(seed=1, prompts=6)
+    shapes = [(m.num_q_heads, m.num_kv_heads, [int(x) for x in m.prompt_lens]) for m in models]
+    shapes.append((16, 2, [300, 5, 129]))
+    shapes.append((8, 8, []))
+    total_blocks = sum(sum((n + bs - 1) // bs for n in lens) * hk for _, hk, lens in shapes)
+    N = total_blocks + 50
+    ids = np.random.Generator(np.random.PCG64(5)).permutation(N)
+    dk_pool, dv_pool = allocate_gpu_cache(N, bs, DEV, dtype=dtype)
+    dk_pool.zero_()
+    dv_pool.zero_()
+    hk_pool, hv_pool = dk_pool.cpu(), dv_pool.cpu()
+    pcalls, wcalls, singles, cur = [], [], [], 0
+    for mi, (Hq, Hkv, lens) in enumerate(shapes):
+        g = torch.Generator().manual_seed(50 + mi)
+        T = sum(lens)
+        pad = (T + 7) // 8 * 8
+        qkv = torch.randn((pad, (Hq + 2 * Hkv) * D), generator=g).to(dtype)
+        dq, dk, dv = qkv.to(DEV).split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+        cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32), device=DEV)
+        fused_out = torch.zeros((pad, Hq * D), dtype=dtype, device=DEV)
+        single_out = torch.zeros_like(fused_out)
+        pcalls.append(ops.PrefillCall(fused_out, dq, dk, dv, cu, lens, D ** -0.5, Hkv))
+        if T:
+            ops.prefill_causal(single_out, dq, dk, dv, cu, max(lens), D ** -0.5, Hkv, prompt_lens=lens)
+            slots, used = workloads.prefill_slot_mapping(lens, Hkv, bs, ids[cur:])
+            cur += used
+            wcalls.append(ops.CacheWriteCall(dk, dv, torch.from_numpy(slots).to(DEV), num_tokens=T))
+            _, k, v = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+            orc.reshape_and_cache(k, v, hk_pool, hv_pool, torch.from_numpy(slots), num_tokens=T)
+        singles.append((fused_out, single_out, T))
+    ops.multi_prefill_causal(pcalls)
+    ops.multi_reshape_and_cache(wcalls, dk_pool, dv_pool)
+    torch.cuda.synchronize()
+    for fused_out, single_out, T in singles:
+        assert torch.equal(fused_out.view(torch.int16), single_out.view(torch.int16))
+        if T:
+            assert single_out[:T].float().abs().sum().item() > 0
+    assert torch.equal(dk_pool.cpu().view(torch.int16), hk_pool.view(torch.int16))
+    assert torch.equal(dv_pool.cpu().view(torch.int16), hv_pool.view(torch.int16))
+
+
+def test_fused_prefill_falls_back_to_one_launch_per_model_when_the_tiles_do_not_fit():
+    """More query tiles than the shared kernel argument lists (here 2 x 520): the
+    call still returns every model's result, identical to the separate calls."""
+    _announce("fused prefill, too many tiles")
+    outs = []
+    calls = []
+    for mi in range(2):
+        g = torch.Generator().manual_seed(70 + mi)
+        lens = [100] * 520
+        T = sum(lens)
+        qkv = torch.randn((T, 3 * D), generator=g).half().to(DEV)
+        q, k, v = qkv.split([D, D, D], dim=-1)
+        cu = torch.arange(0, T + 1, 100, dtype=torch.int32, device=DEV)
+        a, b = torch.zeros((T, D), dtype=torch.float16, device=DEV), torch.zeros((T, D), dtype=torch.float16, device=DEV)
+        calls.append(ops.PrefillCall(a, q, k, v, cu, lens, D ** -0.5, 1))
+        ops.prefill_causal(b, q, k, v, cu, 100, D ** -0.5, 1, prompt_lens=lens)
+        outs.append((a, b))
+    ops.multi_prefill_causal(calls)
+    torch.cuda.synchronize()
+    for a, b in outs:
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16)) and a.float().abs().sum().item() > 0
+
+
 def test_prefill_rejects_bad_arguments():
     q = torch.zeros((8, 256), dtype=torch.float16, device=DEV)
     cu = torch.tensor([0, 8], dtype=torch.int32, device=DEV)
