@@ -61,7 +61,7 @@ def parse():
     ap.add_argument("--unfused", action="store_true", help="one launch per model instead of one fused launch")
     ap.add_argument("--workload", default="mixed3_decode",
                     choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long", "model_ops", "host_step",
-                             "cu_masks", "prefill_long"],
+                             "cu_masks", "prefill_long", "decode_timeline"],
                     help="mixed3_decode is the headline metric; the others are the remaining synthetic "
                          "shapes, each printing its own JSON line")
     return ap.parse_args()
@@ -403,6 +403,81 @@ def bench_cu_masks(args):
                   "kernel": "probe_where_kernel (records XCC_ID / HW_ID per workgroup)"}, dtype="u32")
 
 
+def bench_decode_timeline(args):
+    """Per-phase timeline of one launch of the headline kernel, from the tracing
+    build of the library (libmuxattn_trace.so, `python -m muxserve_amd.build
+    trace`): wave 0 of every workgroup stamps the 100 MHz clock at the ends of
+    its phases.  Prints the phase statistics and the launch in 2 us bins."""
+    import ctypes
+    import torch
+    from muxserve_amd import _lib, ops, workloads
+    from muxserve_amd.build import TRACE_LIB
+    from muxserve_amd.pool import allocate_gpu_cache, num_gpu_blocks
+    if os.path.abspath(_lib.ATTN_LIB_PATH) != os.path.abspath(TRACE_LIB):
+        raise SystemExit("decode_timeline needs the tracing build: python -m muxserve_amd.build trace, then run with "
+                         f"MUXSERVE_ATTN_LIB={TRACE_LIB}")
+    lib = _lib.attn()
+    lib.mux_decode_trace_set.restype = ctypes.c_int32
+    lib.mux_decode_trace_set.argtypes = [ctypes.c_void_p, ctypes.c_int64]
+    dev, bs = "cuda:0", 16
+    N = num_gpu_blocks(args.pool_util, torch.cuda.get_device_properties(0).total_memory, bs)
+    k_pool, v_pool = allocate_gpu_cache(N, bs, dev)
+    sets = []
+    for i in range(3):
+        models, need = workloads.config2(seed=args.seed + 1 + i, num_pool_blocks=N)
+        for j, m in enumerate(models):
+            m.to_device(dev, torch.float16, seed=j)
+        calls = [ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                                total_context_len=int(m.context_lens.sum()),
+                                context_lens_host=None if args.no_host_lens else
+                                torch.from_numpy(np.ascontiguousarray(m.context_lens, dtype=np.int32)))
+                 for m in models]
+        sets.append((models, calls))
+    rows = 20000
+    table = torch.zeros((rows, 8), dtype=torch.int64, device=dev)
+    for i in range(12):
+        ops.multi_decode(sets[i % 3][1], k_pool, v_pool)
+    torch.cuda.synchronize()
+    ops.multi_decode(sets[1][1], k_pool, v_pool)            # a launch right before, as in the benchmark loop
+    assert lib.mux_decode_trace_set(table.data_ptr(), rows) == 0
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    ops.multi_decode(sets[0][1], k_pool, v_pool)
+    e1.record()
+    torch.cuda.synchronize()
+    lib.mux_decode_trace_set(None, 0)
+    t = table.cpu().numpy()
+    t = t[t[:, 6] > 0]
+    t0 = t[:, 0].min()
+    us = lambda x: (x - t0) / 100.0                                                    # noqa: E731
+    a, b, c, d, e, f, g = (us(t[:, i]) for i in range(7))
+    ntok, split = t[:, 7] & 0xffff, (t[:, 7] >> 16) & 1
+    stats = {}
+    for name, x, y in (("entry_to_unit_known", a, b), ("unit_known_to_ids_and_q", b, c), ("ids_and_q_to_kv_issued", c, d),
+                       ("kv_issued_to_consumed", d, e), ("consumed_to_barrier", e, f), ("barrier_to_done", f, g),
+                       ("life", a, g)):
+        dd = y - x
+        stats[name] = {"mean": float(dd.mean()), "p50": float(np.median(dd)), "p90": float(np.percentile(dd, 90))}
+    bins = []
+    for lo in np.arange(0.0, float(g.max()) + 2.0, 2.0):
+        mid = lo + 1.0
+        bins.append({"t_us": float(lo), "started": int(((a >= lo) & (a < lo + 2)).sum()),
+                     "alive": int(((a <= mid) & (g > mid)).sum()), "kv_in_flight": int(((c <= mid) & (e > mid)).sum()),
+                     "MB_consumed": float(ntok[(e >= lo) & (e < lo + 2)].sum() * 512 / 1e6)})
+    first = slice(0, 768)
+    cfg = {"workload": "decode_timeline", "kernel_ms_with_stamps": e0.elapsed_time(e1), "span_us": float(g.max()),
+           "workgroups": int(len(t)), "MB": float(ntok.sum() * 512 / 1e6), "phases_us": stats,
+           "split_units": {"n": int(split.sum()), "barrier_to_done_mean_us": float((g - f)[split == 1].mean())},
+           "single_units": {"n": int((split == 0).sum()), "barrier_to_done_mean_us": float((g - f)[split == 0].mean())},
+           "first_768_workgroups_mean_us": {"entry": float(a[first].mean()), "unit_known": float(b[first].mean()),
+                                            "ids_and_q": float(c[first].mean()), "kv_issued": float(d[first].mean()),
+                                            "consumed": float(e[first].mean())},
+           "bins_2us": bins}
+    return _line("decode kernel per-phase timeline (tracing build)", float(g.max()), "us", args, float(g.max()) * 1e-3, cfg,
+                 {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": None, "traffic": None,
+                  "kernel": "paged_decode_kernel<F16,16,1,4> with phase stamps"}, higher=False)
+
+
 def bench_gqa_long(args):
     """Config 5: 64 query heads over 8 kv heads, bf16, batch 64, ctx U[2048, 8192]."""
     import torch
@@ -673,7 +748,7 @@ def main():
         print("bench.py: this build runs on one GPU only (no collectives or sharding); use --gpus 1",
               file=sys.stderr)
         sys.exit(2)
-    other = {"prefill3": bench_prefill3, "cache_write": bench_cache_write, "colocated": bench_colocated, "cu_masks": bench_cu_masks, "prefill_long": bench_prefill_long,
+    other = {"prefill3": bench_prefill3, "cache_write": bench_cache_write, "colocated": bench_colocated, "cu_masks": bench_cu_masks, "prefill_long": bench_prefill_long, "decode_timeline": bench_decode_timeline,
              "gqa_long": bench_gqa_long, "model_ops": bench_model_ops, "host_step": bench_host_step}
     if args.workload in other:
         print(json.dumps(other[args.workload](args)))

@@ -4,6 +4,10 @@
     libmuxattn.so  - hipcc, gfx950 kernels + their C ABI
     libmuxtorch.so - g++,   thin TORCH_LIBRARY operators over libmuxattn.so's C ABI
     libmuxprobe.so - hipcc, a bare gather-read kernel: bench.py's yardstick, not product
+    libmuxattn_trace.so - hipcc, libmuxattn.so built with -DMUX_TRACE (per-workgroup phase
+                     stamps in the decode kernel) for `bench.py --workload decode_timeline`;
+                     built on request only (`python -m muxserve_amd.build trace`), never loaded
+                     by the package
 
 Run as ``python -m muxserve_amd.build``.  Nothing here runs at import time of
 the package: the loaders in muxserve_amd._lib only open what this step built
@@ -22,6 +26,7 @@ HOST_LIB = os.path.join(PKG, "libmuxhost.so")
 ATTN_LIB = os.path.join(PKG, "libmuxattn.so")
 TORCH_LIB = os.path.join(PKG, "libmuxtorch.so")
 PROBE_LIB = os.path.join(PKG, "libmuxprobe.so")
+TRACE_LIB = os.path.join(PKG, "libmuxattn_trace.so")
 PROBE_SOURCES = [os.path.join(CSRC, "probe", "probe.hip")]
 TORCH_SOURCES = [os.path.join(CSRC, "torch", "mux_torch_ops.cpp")]
 
@@ -56,6 +61,12 @@ def build_hip(extra=()):
     return ATTN_LIB
 
 
+def build_trace():
+    srcs = [s for s in HIP_SOURCES if os.path.exists(s)]
+    _run([HIPCC, *HIP_FLAGS, "-DMUX_TRACE", f"-I{INCLUDE}", f"-I{os.path.join(CSRC, 'hip')}", *srcs, "-o", TRACE_LIB])
+    return TRACE_LIB
+
+
 def build_probe():
     _run([HIPCC, *HIP_FLAGS, f"-I{os.path.join(CSRC, 'probe')}", *PROBE_SOURCES, "-o", PROBE_LIB])
     return PROBE_LIB
@@ -86,4 +97,5 @@ def build_all():
 
 if __name__ == "__main__":
     what = sys.argv[1] if len(sys.argv) > 1 else "all"
-    {"host": build_host, "hip": build_hip, "torch": build_torch, "probe": build_probe, "all": build_all}[what]()
+    {"host": build_host, "hip": build_hip, "torch": build_torch, "probe": build_probe, "trace": build_trace,
+     "all": build_all}[what]()

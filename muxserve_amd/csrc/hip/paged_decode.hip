@@ -41,6 +41,30 @@ namespace mux {
 
 thread_local int32_t g_last_hip_error = 0;
 
+// Tracing build (-DMUX_TRACE, libmuxattn_trace.so; never the shipped library):
+// wave 0 of every workgroup of the vector-ALU decode kernel stamps the 100 MHz
+// clock at the ends of its phases into a caller-provided table, 8 int64 per
+// workgroup: [0] entry, [1] unit known, [2] block ids and q there, [3] K/V loads
+// of the (last) tile issued, [4] tile consumed, [5] past the workgroup's barrier,
+// [6] merge / publish / combine done, [7] tokens of the unit | split << 16.
+#ifdef MUX_TRACE
+__device__ long long *g_decode_trace = nullptr;
+__device__ long long g_decode_trace_rows = 0;
+#define MUX_TR(slot)                                                                         \
+  do {                                                                                       \
+    if (threadIdx.x == 0 && g_decode_trace && blockIdx.x < g_decode_trace_rows)              \
+      g_decode_trace[blockIdx.x * 8 + (slot)] = __builtin_amdgcn_s_memrealtime();            \
+  } while (0)
+#define MUX_TRV(slot, v)                                                                     \
+  do {                                                                                       \
+    if (threadIdx.x == 0 && g_decode_trace && blockIdx.x < g_decode_trace_rows)              \
+      g_decode_trace[blockIdx.x * 8 + (slot)] = (v);                                         \
+  } while (0)
+#else
+#define MUX_TR(slot)
+#define MUX_TRV(slot, v)
+#endif
+
 constexpr int kWavesPerGroup = 4;         // waves cooperating on one unit
 
 struct DecodeItemDev {
@@ -629,14 +653,22 @@ __device__ __forceinline__ void fetch_q(const DecodeItemDev &I, int seq, int hq0
   }
 }
 
+#ifdef MUX_TRACE
+// (the stamps cost two registers; the tracing build is held to the shipped kernel's
+// three waves per SIMD so that the timeline is that of the same residency)
+#define MUX_DECODE_BOUNDS __launch_bounds__(64 * NW, G == 1 ? 3 : 1)
+#else
+#define MUX_DECODE_BOUNDS __launch_bounds__(64 * NW)
+#endif
 template <typename T, int BS, int G, int NW>
-__global__ __launch_bounds__(64 * NW) void paged_decode_kernel(const DecodeParams P) {
+__global__ MUX_DECODE_BOUNDS void paged_decode_kernel(const DecodeParams P) {
   using Geo = Geometry<BS>;
   __shared__ __attribute__((aligned(16))) float p_lds[NW][G][64];     // per-wave probabilities of a tile
   __shared__ __attribute__((aligned(16))) uint32_t q_lds[NW][G][64];  // G > 1: per-wave copy of the group's q
   __shared__ float x_acc[NW][G][kHeadSize];                           // per-wave partial outputs
   __shared__ float x_ml[NW][G][2];
 
+  MUX_TR(0);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int w = blockIdx.x;
@@ -657,6 +689,8 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_kernel(const DecodeParam
   if (!locate_pair(P, I, partition, e, lane, u.seq, u.split, u.ctx)) return;
   u.t0 = u.split * partition;
   u.t1 = min(u.ctx, u.t0 + partition);
+  MUX_TR(1);
+  MUX_TRV(7, static_cast<long long>(u.t1 - u.t0) | (static_cast<long long>(u.ctx > partition) << 16));
   const int hq0 = u.wh * G;
   const int hk = hq0 / I.ratio;
 
@@ -673,6 +707,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_kernel(const DecodeParam
   int id_next = load_block_id<BS>(trow, tb0, u.t1, lane, P.last_block);
   uint32_t q_s[64];
   fetch_q<G>(I, u.seq, hq0, lane, q_s, q_lds[wave]);
+  MUX_TR(2);
 
   float m[G], l[G], acc[G][Geo::VI];
 #pragma unroll
@@ -688,12 +723,16 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_kernel(const DecodeParam
     uint4 kreg[16];
     uint4 vreg[Geo::BPT][Geo::VI];
     issue_tile_loads<BS>(kreg, vreg, kpool, vpool, id, tb, u.t1, lane);
+    MUX_TR(3);
     consume_tile<T, BS, G>(kreg, vreg, q_s, q_lds[wave], p_lds[wave], m, l, acc, I.scale_log2, tb, u.t1, lane);
+    MUX_TR(4);
   }
   stash_wave_partial<BS, G>(m, l, acc, x_acc[wave], x_ml[wave], lane);
   __syncthreads();
+  MUX_TR(5);
   if (wave != 0) return;
   merge_and_write<T, G, NW>(I, u, partition, x_acc, x_ml, n_active, lane);
+  MUX_TR(6);
 }
 
 // ---------------------------------------------------------------------------
@@ -1442,3 +1481,15 @@ int32_t mux_paged_decode(void *out, int64_t out_row_stride, const void *q, int64
 }
 
 }  // extern "C"
+
+#ifdef MUX_TRACE
+// Tracing build only: where the decode kernel's workgroups write their stamps
+// (DEVICE int64 [rows, 8], zero-filled by the caller; NULL switches it off).
+extern "C" int32_t mux_decode_trace_set(void *table, int64_t rows) {
+  long long *p = static_cast<long long *>(table);
+  long long n = table ? rows : 0;
+  MUX_HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(mux::g_decode_trace), &p, sizeof(p)));
+  MUX_HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(mux::g_decode_trace_rows), &n, sizeof(n)));
+  return MUXA_OK;
+}
+#endif
