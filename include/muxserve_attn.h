@@ -94,7 +94,14 @@ int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t kv_row_strid
  * the grid, device values above it are clamped.
  * total_context_len: optional host-side upper bound on the sum of
  * context_lens (the serving loop has them on the host before the copy,
- * llm_runtime.py:311-326); it only tightens the grid, 0 = unknown.
+ * llm_runtime.py:311-326); it only tightens the grid, 0 = unknown.  It MUST be
+ * an upper bound: the grid is sized from it, units are enumerated remainders
+ * first, full partitions next, single-partition sequences last, and units
+ * beyond the grid are not run - an understated sum first leaves outputs of
+ * single-partition sequences unwritten and, beyond those, leaves arrival
+ * counters of split sequences non-zero, after which the workspace has to be
+ * re-initialised (mux_paged_decode_workspace_init) before its next use.  With
+ * context_lens_host the enumeration is exact and this field is not used.
  * context_lens_host: optional HOST copy of context_lens [num_seqs] (same
  * place in the serving loop, llm_runtime.py:311-326: the lengths are a host
  * list before they become a tensor).  When every model of a launch comes with

@@ -194,7 +194,7 @@ def test_fresh_cu_resource_closed_forms():
 @pytest.mark.parametrize("num_cus", [256, 304, 64])
 def test_part_masks_are_disjoint_cover_the_gpu_and_are_balanced_over_the_dies(num_cus):
     """Mask bit i enables a compute unit of die i % 8 (consecutive bits go
-    round-robin over the 8 accelerator dies: measured, profiles/cu_mask_*).
+    round-robin over the 8 accelerator dies: measured with a kernel that records the die of every workgroup).
     Every part must therefore hold floor or ceil of its share of every die,
     parts must not overlap and all ten together are the whole GPU."""
     seen = set()
