@@ -381,6 +381,61 @@ void prefill_causal(at::Tensor out, const at::Tensor &q, const at::Tensor &k, co
         "mux_prefill_causal");
 }
 
+// The prompts of several colocated models in one launch: element i of every
+// list describes model i.  prompt_lens_host: CPU int32 [P_i] per model (the
+// reference holds them on the host, InputMetadata.prompt_lens), or an empty
+// list when none is given.
+void multi_prefill_causal(at::TensorList outs, at::TensorList qs, at::TensorList ks, at::TensorList vs,
+                          at::TensorList cu_seqlens, at::TensorList prompt_lens_host, at::IntArrayRef max_prompt_lens,
+                          at::ArrayRef<double> scales, at::IntArrayRef num_kv_heads) {
+  const size_t n = outs.size();
+  TORCH_CHECK(n >= 1 && n <= MUXA_MAX_DECODE_ITEMS && qs.size() == n && ks.size() == n && vs.size() == n &&
+                  cu_seqlens.size() == n && max_prompt_lens.size() == n && scales.size() == n &&
+                  num_kv_heads.size() == n && (prompt_lens_host.empty() || prompt_lens_host.size() == n),
+              "multi_prefill_causal: 1..", MUXA_MAX_DECODE_ITEMS, " models, one entry per model in every list");
+  MuxPrefillItem items[MUXA_MAX_DECODE_ITEMS];
+  for (size_t i = 0; i < n; ++i) {
+    const at::Tensor &out = outs[i], &q = qs[i], &k = ks[i], &v = vs[i], &cu = cu_seqlens[i];
+    need_gpu({&out, &q, &k, &v, &cu});
+    TORCH_CHECK(cu.scalar_type() == at::kInt && cu.dim() == 1 && cu.is_contiguous() && cu.size(0) >= 1,
+                "cu_seqlens: expected contiguous int32 [P+1]");
+    const int64_t P = cu.size(0) - 1;
+    TORCH_CHECK(q.dim() == 2 && q.size(1) % kHead == 0 && k.dim() == 2 && k.size(1) == num_kv_heads[i] * kHead &&
+                    k.sizes() == v.sizes(),
+                "q [T, Hq*128], k/v [T, Hkv*128] expected");
+    TORCH_CHECK(q.scalar_type() == qs[0].scalar_type() && q.scalar_type() == k.scalar_type() &&
+                    k.scalar_type() == v.scalar_type() && v.scalar_type() == out.scalar_type(),
+                "q, k, v, out of all models must share one dtype");
+    const int64_t kv_stride = rows(k, "k");
+    TORCH_CHECK(rows(v, "v") == kv_stride, "k and v row strides differ");
+    MuxPrefillItem &it = items[i];
+    it = MuxPrefillItem{};
+    it.out = out.data_ptr();
+    it.out_row_stride = rows(out, "out");
+    it.q = q.data_ptr();
+    it.q_row_stride = rows(q, "q");
+    it.k = k.data_ptr();
+    it.v = v.data_ptr();
+    it.kv_row_stride = kv_stride;
+    it.cu_seqlens = cu.data_ptr<int32_t>();
+    it.prompt_lens_host = nullptr;
+    if (!prompt_lens_host.empty()) {
+      const at::Tensor &h = prompt_lens_host[i];
+      TORCH_CHECK(h.device().is_cpu() && h.scalar_type() == at::kInt && h.dim() == 1 && h.is_contiguous() &&
+                      h.size(0) == P,
+                  "prompt_lens_host: expected a contiguous CPU int32 tensor with one length per prompt");
+      it.prompt_lens_host = h.data_ptr<int32_t>();
+    }
+    it.num_prompts = static_cast<int32_t>(P);
+    it.max_prompt_len = static_cast<int32_t>(max_prompt_lens[i]);
+    it.num_q_heads = static_cast<int32_t>(q.size(1) / kHead);
+    it.num_kv_heads = static_cast<int32_t>(num_kv_heads[i]);
+    it.scale = static_cast<float>(scales[i]);
+  }
+  check(mux_multi_prefill_causal(items, static_cast<int32_t>(n), kHead, dtype_code(qs[0]), stream_of(qs[0])),
+        "mux_multi_prefill_causal");
+}
+
 at::Tensor rms_norm(const at::Tensor &x, const at::Tensor &weight, double eps) {
   need_gpu({&x, &weight});
   TORCH_CHECK(x.dim() == 2 && weight.dim() == 1 && weight.size(0) == x.size(1) &&
@@ -422,6 +477,8 @@ TORCH_LIBRARY(muxserve_amd, m) {
         "int total_context_len, Tensor(b!) workspace, Tensor? context_lens_host=None) -> ()");
   m.def("prefill_causal(Tensor(a!) out, Tensor q, Tensor k, Tensor v, Tensor cu_seqlens, int[] prompt_lens, "
         "int max_prompt_len, float scale, int num_kv_heads) -> ()");
+  m.def("multi_prefill_causal(Tensor(a!)[] outs, Tensor[] qs, Tensor[] ks, Tensor[] vs, Tensor[] cu_seqlens, "
+        "Tensor[] prompt_lens_host, int[] max_prompt_lens, float[] scales, int[] num_kv_heads) -> ()");
   m.def("multi_decode_workspace_bytes(Tensor[] outs, Tensor[] qs, Tensor[] block_tables, Tensor[] context_lens, "
         "int[] max_context_lens, int partition_size) -> int");
   m.def("multi_decode(Tensor(a!)[] outs, Tensor[] qs, Tensor k_pool, Tensor v_pool, Tensor[] block_tables, "
@@ -442,6 +499,7 @@ TORCH_LIBRARY_IMPL(muxserve_amd, CUDA, m) {
   m.impl("paged_decode_workspace_bytes", &paged_decode_workspace_bytes);
   m.impl("paged_decode", &paged_decode);
   m.impl("prefill_causal", &prefill_causal);
+  m.impl("multi_prefill_causal", &multi_prefill_causal);
   m.impl("multi_decode_workspace_bytes", &multi_decode_workspace_bytes);
   m.impl("multi_decode", &multi_decode);
   m.impl("rotary_neox", &rotary_neox);

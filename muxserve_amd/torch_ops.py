@@ -22,7 +22,8 @@ TORCH_LIB_PATH = os.environ.get("MUXSERVE_TORCH_LIB", os.path.join(_PKG, "libmux
 
 OPERATORS = ("reshape_and_cache", "rope_reshape_and_cache", "multi_reshape_and_cache", "rotary_neox",
              "paged_decode_workspace_bytes",
-             "paged_decode", "multi_decode_workspace_bytes", "multi_decode", "prefill_causal", "rms_norm",
+             "paged_decode", "multi_decode_workspace_bytes", "multi_decode", "prefill_causal",
+             "multi_prefill_causal", "rms_norm",
              "silu_and_mul", "greedy_sample_workspace_bytes", "greedy_sample")
 
 _loaded = False
@@ -71,6 +72,17 @@ def prefill_causal(out, q, k, v, cu_seqlens, max_prompt_len: int, scale: float, 
                    prompt_lens=None) -> None:
     load().prefill_causal(out, q, k, v, cu_seqlens, [] if prompt_lens is None else [int(x) for x in prompt_lens],
                           int(max_prompt_len), float(scale), int(num_kv_heads))
+
+
+def multi_prefill_causal(calls) -> None:
+    """Causal prefill of several colocated models' prompts in one launch.  `calls`:
+    muxserve_amd.ops.PrefillCall objects (out, q, k, v, cu_seqlens, prompt_lens,
+    scale, num_kv_heads), one per model."""
+    lens = [torch.tensor([int(x) for x in c.prompt_lens], dtype=torch.int32) for c in calls]
+    load().multi_prefill_causal([c.out for c in calls], [c.q for c in calls], [c.k for c in calls],
+                                [c.v for c in calls], [c.cu_seqlens for c in calls], lens,
+                                [int(t.max()) if t.numel() else 0 for t in lens], [float(c.scale) for c in calls],
+                                [int(c.num_kv_heads) for c in calls])
 
 
 def paged_decode(out, q, k_pool, v_pool, block_tables, context_lens, max_context_len: int, scale: float,

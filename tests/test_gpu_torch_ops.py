@@ -140,6 +140,38 @@ def test_torch_operators_equal_the_ctypes_path(dtype):
     assert torch.equal(_bits(T.silu_and_mul(x)), _bits(ops.silu_and_mul(x)))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_prefill_operator_equals_the_ctypes_path(dtype):
+    """torch.ops.muxserve_amd.multi_prefill_causal (three models of different head
+    counts, one of them grouped-query, one without prompts) against
+    muxserve_amd.ops.multi_prefill_causal: the same C entry point, bitwise equal."""
+    print(f"[case] fused prefill operator {dtype}", flush=True)
+    shapes = [(4, 4, [70, 1, 200]), (8, 2, [129, 33]), (2, 2, [])]
+    via_ops, via_torch = [], []
+    for mi, (Hq, Hkv, lens) in enumerate(shapes):
+        g = torch.Generator().manual_seed(90 + mi)
+        T_ = sum(lens)
+        pad = (T_ + 7) // 8 * 8
+        qkv = torch.randn((pad, (Hq + 2 * Hkv) * D), generator=g).to(dtype).to(DEV)
+        q, k, v = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+        cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32), device=DEV)
+        for calls in (via_ops, via_torch):
+            calls.append(ops.PrefillCall(torch.zeros((pad, Hq * D), dtype=dtype, device=DEV), q, k, v, cu, lens,
+                                         D ** -0.5, Hkv))
+    ops.multi_prefill_causal(via_ops)
+    torch_ops.multi_prefill_causal(via_torch)
+    torch.cuda.synchronize()
+    for a, b, (_, _, lens) in zip(via_ops, via_torch, shapes):
+        assert torch.equal(_bits(a.out), _bits(b.out))
+        if lens:
+            assert a.out[:sum(lens)].float().abs().sum().item() > 0
+    # one list shorter than the others is refused
+    T = torch_ops.load()
+    c = via_torch[0]
+    with pytest.raises(RuntimeError):
+        T.multi_prefill_causal([c.out], [c.q], [c.k], [c.v], [c.cu_seqlens], [], [200], [1.0, 1.0], [4])
+
+
 def test_torch_operators_refuse_bad_arguments():
     print("[case] torch operators, bad arguments", flush=True)
     T = torch_ops.load()
