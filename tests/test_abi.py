@@ -85,3 +85,34 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
                        timeout=120)
     assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_grid_bound_from_the_context_sum_covers_every_pair():
+    """The host-side sum of context lengths tightens the number of (sequence,
+    partition) pairs a launch reserves.  The reservation is visible, without a
+    GPU, in the workspace size of a batch large enough to need a pair table
+    (16 bytes per reserved pair): for random batches it must never be smaller
+    than the true number of pairs, and never looser than floor(sum / partition)
+    + sequences (the table is rounded up to 256 bytes = 16 pairs)."""
+    import numpy as np
+    lib = _lib.attn()
+    rng = np.random.Generator(np.random.PCG64(11))
+    for partition in (64, 256, 512):
+        for trial in range(20):
+            B = 16 * int(rng.integers(17, 40))      # a multiple of 16: the loose table has no rounding pad
+            hi = int(rng.choice([partition // 2, partition, 3 * partition, 2000]))
+            ctx = rng.integers(0, hi + 1, size=B).astype(np.int64)
+            it = _lib.MuxDecodeItem()
+            it.num_seqs, it.num_q_heads, it.num_kv_heads = B, 4, 4
+            it.num_layers, it.layer = 1, 0
+            it.max_context_len = int(ctx.max())
+            it.max_blocks = (it.max_context_len + 15) // 16
+            it.total_context_len = 0
+            loose = lib.mux_paged_decode_workspace_bytes(ctypes.addressof(it), 1, partition)
+            it.total_context_len = int(ctx.sum())
+            tight = lib.mux_paged_decode_workspace_bytes(ctypes.addressof(it), 1, partition)
+            max_splits = max(1, -(-it.max_context_len // partition))
+            reserved = B * max_splits - (loose - tight) // 16          # pairs reserved with the hint, rounded up to 16
+            true_pairs = int((-(-ctx // partition)).sum())
+            assert reserved >= true_pairs, (partition, trial, reserved, true_pairs)
+            assert reserved <= min(B * max_splits, int(ctx.sum()) // partition + B) + 15
