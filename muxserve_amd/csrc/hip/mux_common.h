@@ -125,6 +125,30 @@ __device__ __forceinline__ float wave_sum(float v) {
   return (lane_bcast(v, 0) + lane_bcast(v, 16)) + (lane_bcast(v, 32) + lane_bcast(v, 48));
 }
 
+// A lane's value combined with that of lane ^ 32 (lane ^ 16), on the vector ALU:
+// v_permlane32_swap exchanges the upper half of one register with the lower
+// half of another (v_permlane16_swap: the odd 16-lane rows of one with the even
+// rows of the other), so with the same value in both, every lane ends up with
+// its own half's value in one result and the other half's in the other.  The
+// usual __shfl_xor is a ds_bpermute, which queues behind the LDS traffic of the
+// whole compute unit.
+__device__ __forceinline__ float max_with_lane_xor32(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_with_lane_xor32(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float max_with_lane_xor16(float v) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_with_lane_xor16(float v) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Blocks this wave until every vector-memory access it has issued - loads AND
 // stores - has completed (on gfx9 stores count in vmcnt and are acknowledged
 // once they have reached the level their scope bits name).  A workgroup-scope

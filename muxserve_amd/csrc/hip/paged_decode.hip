@@ -932,8 +932,7 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
         sacc[tg][i] = sc;
         mx = fmaxf(mx, sc);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));  // the step has at least one valid token: finite
+    mx = max_with_lane_xor32(max_with_lane_xor16(mx));   // the step has at least one valid token: finite
     const float m_new = fmaxf(m, mx);
     const float alpha = fast_exp2(m - m_new);
     float psum = 0.f;
@@ -1012,8 +1011,7 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
   }
 
   // ---- this wave's partial to LDS, in the layout the merge expects ----------------------
-  l += __shfl_xor(l, 16);
-  l += __shfl_xor(l, 32);
+  l = sum_with_lane_xor32(sum_with_lane_xor16(l));
   if (h < G) {
 #pragma unroll
     for (int nb = 0; nb < 8; ++nb)

@@ -318,7 +318,7 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
     for (int kb = 0; kb < kNKB; ++kb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kb][i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    mx = max_with_lane_xor32(mx);
     const float m_new = fmaxf(m_run, mx);
     // Rows past the prompt may have no valid key at all; keep them finite.
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
@@ -413,7 +413,7 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
   }
 
   // ---- normalise and store: register i of block mb is d = 32 mb + 8 (i/4) + 4 half + i%4 ------
-  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float l_tot = sum_with_lane_xor32(l_run);
   const float inv = 1.f / l_tot;
   if (I.out_rows_16b) {
     // Through LDS, so that the rows go out as whole 256-byte runs (16 bytes per
