@@ -319,10 +319,28 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
 #pragma unroll
       for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kb][i]);
     mx = max_with_lane_xor32(mx);
-    const float m_new = fmaxf(m_run, mx);
-    // Rows past the prompt may have no valid key at all; keep them finite.
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float neg_m = -m_use * I.scale_log2;
+    // The reference of the exponents (m_run) only moves when some row's maximum has
+    // risen more than kRescaleStep (in the exponent's units) above it - and on the
+    // wave's first tile, to that tile's maximum: probabilities then reach
+    // 2^kRescaleStep at most, and the 64 accumulators and the running sum are
+    // rescaled rarely instead of whenever a maximum rises at all (with 32 rows per
+    // wave, that is in most tiles of a prompt's first hundreds of keys).
+    constexpr float kRescaleStep = 8.f;
+    const bool move = m_run == -INFINITY ? mx != -INFINITY : (mx - m_run) * I.scale_log2 > kRescaleStep;
+    if (__builtin_amdgcn_ballot_w64(move) != 0) {
+      const float m_new = fmaxf(m_run, mx);
+      // Rows past the prompt may have no valid key at all; keep them finite.
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = fast_exp2((m_run - m_use) * I.scale_log2);
+      l_run *= alpha;
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[mb][i] *= alpha;
+      m_run = m_use;
+    }
+    // (a row that has not seen a valid key yet keeps a finite reference)
+    const float neg_m = m_run == -INFINITY ? 0.f : -m_run * I.scale_log2;
     float psum = 0.f;
     Frag pf[2 * kNKB];                          // B fragments: [kb][step] -> index 2 kb + st
     // bf16 keeps only 8 mantissa bits of a probability, which alone would cost
@@ -355,18 +373,7 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
         }
       }
     }
-    // The running max rises only in the first tiles of a row; skip the rescale
-    // of the 64 accumulators when no lane of the wave needs it.
-    if (__builtin_amdgcn_ballot_w64(m_use > m_run) != 0) {
-      const float alpha = fast_exp2((m_run - m_use) * I.scale_log2);
-      l_run *= alpha;
-#pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) oacc[mb][i] *= alpha;
-    }
     l_run += psum;
-    m_run = m_use;
 
     // ---- O^T += V^T . P^T ---------------------------------------------------------------
     // k-slot j of lane half h in step (kb, st) is key 32 kb + 16 st + 8 (j/4) + 4 h + j%4
