@@ -310,6 +310,44 @@ def test_fused_prefill_falls_back_to_one_launch_per_model_when_the_tiles_do_not_
         assert torch.equal(a.view(torch.int16), b.view(torch.int16)) and a.float().abs().sum().item() > 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_prefill_row_maxima_that_jump_far_above_the_softmax_reference(dtype):
+    """The kernel keeps the reference of its exponents until some row's maximum
+    has risen by more than 8 (in the exponent) above it.  N(0,1) data never gets
+    there after the first tile, so here the scores are made to jump: all queries
+    share a strong component along one direction and a few keys, later and later
+    in the prompt, point along it with growing length - the running maximum of
+    every row then rises by 10 to 20 at those keys (several moves of the
+    reference per wave, in different tiles), while the rows before a spike keep
+    an ordinary mixture.  A second prompt has its spike in the very first tile."""
+    _announce(f"prefill softmax reference moves {dtype}")
+    Hq = Hkv = 2
+    lens = [700, 190]
+    g = torch.Generator().manual_seed(77)
+    T = sum(lens)
+    pad = (T + 7) // 8 * 8
+    u = torch.randn((Hq, D), generator=g)
+    u = u / u.norm(dim=-1, keepdim=True)
+    q = torch.randn((pad, Hq, D), generator=g) + 4.0 * u
+    k = torch.randn((pad, Hkv, D), generator=g)
+    v = torch.randn((pad, Hkv, D), generator=g)
+    for pos, beta in ((40, 20.0), (300, 45.0), (301, 44.0), (650, 80.0), (700 + 3, 30.0), (700 + 150, 60.0)):
+        k[pos] = beta * u
+    q, k, v = (x.reshape(pad, -1).to(dtype) for x in (q, k, v))
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32, device=DEV)
+    out = torch.zeros((pad, Hq * D), dtype=dtype, device=DEV)
+    ops.prefill_causal(out, q.to(DEV), k.to(DEV), v.to(DEV), cu, max(lens), D ** -0.5, Hkv, prompt_lens=lens)
+    torch.cuda.synchronize()
+    got = out.float().cpu()[:T]
+    want = orc.prefill_causal(q, k, v, lens, D ** -0.5, Hkv)
+    assert torch.isfinite(got).all()
+    # the scores really jump: the spike keys dominate the rows after them
+    s_spike = (q[651].float().reshape(Hq, D) * k[650].float().reshape(Hkv, D)).sum(-1) * D ** -0.5 * 1.4427
+    assert (s_spike > 20).all()
+    excess = ((got - want).abs() - _bound(want, dtype)).max().item()
+    assert excess <= 0, f"max-abs error {(got - want).abs().max().item():.3e}"
+
+
 def test_prefill_rejects_bad_arguments():
     q = torch.zeros((8, 256), dtype=torch.float16, device=DEV)
     cu = torch.tensor([0, 8], dtype=torch.int32, device=DEV)
