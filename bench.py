@@ -785,13 +785,15 @@ def main():
         sets.append((models, calls, torch.from_numpy(used.astype(np.int32)).to(dev)))
     torch.cuda.synchronize()
 
+    # Every batch's launch is prepared once (tensor checks, descriptors, workspace): a step is
+    # then a single call into the C ABI, as in a serving loop that runs the same step shape
+    # layer after layer.
+    launches = [[ops.DecodeLaunch([c], k_pool, v_pool, args.partition) for c in calls] if args.unfused
+                else [ops.DecodeLaunch(calls, k_pool, v_pool, args.partition)] for _, calls, _ in sets]
+
     def step(i):
-        calls = sets[i % len(sets)][1]
-        if args.unfused:
-            for c in calls:
-                ops.multi_decode([c], k_pool, v_pool, partition_size=args.partition)
-        else:
-            ops.multi_decode(calls, k_pool, v_pool, partition_size=args.partition)
+        for launch in launches[i % len(launches)]:
+            launch()
 
     for i in range(args.warmup):
         step(i)
@@ -801,11 +803,27 @@ def main():
     ev0.record()
     for i in range(args.steps):
         step(i)
+    t_enq = time.perf_counter()
     ev1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    enqueue_us = (t_enq - t0) * 1e6 / args.steps
     ev_ms = ev0.elapsed_time(ev1) / args.steps
     ms = max(wall_ms, ev_ms)
+
+    # Outside the timed region: every batch's launch on its own between two events (a
+    # launch with nothing queued behind it: kernel plus the dispatch latency around it).
+    singles = []
+    for r in range(3):
+        for i in range(len(sets)):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            a.record()
+            step(i)
+            b.record()
+            b.synchronize()
+            singles.append((i, a.elapsed_time(b) * 1e3))
+    single_us = [float(np.median([t for j, t in singles if j == i])) for i in range(len(sets))]
 
     # The yardstick: the same blocks read by the bare gather-read probe (the decode
     # kernel's loads, no table walk, no arithmetic), same rotation of the sets.
@@ -852,6 +870,11 @@ def main():
             "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiles/paged_decode_mixed3_hbm_traffic.txt",
             "kernel": "paged_decode_kernel<F16,16,1,4>",
             "event_ms_per_step": ev_ms,
+            "wall_ms_per_step": wall_ms,
+            "host_enqueue_us_per_step": enqueue_us,
+            "units_enumerated_on_the_host": [[l.host_pairs for l in ls] for ls in launches],
+            "single_launch_event_us_per_batch": single_us,
+            "single_launch_event_us_weighted_mean": float(sum(t * v for t, v in zip(single_us, [len(range(i, args.steps, len(sets))) for i in range(len(sets))])) / args.steps),
             "bare_gather_read_of_the_same_blocks": {
                 "ms": probe_ms, "bytes": int(probe_bytes), "GB/s": probe_bytes / (probe_ms * 1e-3) / 1e9,
                 "kernel": "probe_gather_read_kernel (whole 4 KiB blocks, no arithmetic)"},

@@ -145,6 +145,13 @@ typedef struct MuxDecodeItem {
 size_t mux_paged_decode_workspace_bytes(const MuxDecodeItem *items, int32_t n_items,
                                         int32_t partition_size);
 
+/* How many (sequence, unit) pairs a mux_multi_decode call with these items
+ * would enumerate on the host and carry in the kernel argument (its first
+ * launch group); 0: the units of that call are enumerated on the device (no
+ * context_lens_host, or more pairs than the argument holds).  Host arithmetic
+ * only, no device needed.  No reference counterpart. */
+int32_t mux_paged_decode_host_pairs(const MuxDecodeItem *items, int32_t n_items, int32_t partition_size);
+
 /* Zero-fills the counter region of a decode workspace (a fill kernel on
  * `stream`, safe to capture). */
 int32_t mux_paged_decode_workspace_init(void *workspace, size_t workspace_bytes, void *stream);

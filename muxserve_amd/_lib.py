@@ -145,6 +145,7 @@ ATTN_SIGNATURES = {
     "mux_multi_prefill_causal": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_vp]),
     "mux_multi_rope_reshape_and_cache": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_vp]),
     "mux_paged_decode_workspace_bytes": (c_sz, [c_vp, c_i32, c_i32]),
+    "mux_paged_decode_host_pairs": (c_i32, [c_vp, c_i32, c_i32]),
     "mux_paged_decode_workspace_init": (c_i32, [c_vp, c_sz, c_vp]),
     "mux_multi_decode": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_i32,
                                  c_vp, c_sz, c_vp]),

@@ -54,17 +54,29 @@ def build_host():
     return HOST_LIB
 
 
+def _compile_and_link(out, extra=(), tag="o"):
+    """One hipcc -c per translation unit, side by side (they are independent:
+    -fno-gpu-rdc), then one link step."""
+    from concurrent.futures import ThreadPoolExecutor
+    objdir = os.path.join(CSRC, "build")
+    os.makedirs(objdir, exist_ok=True)
+    flags = [f for f in HIP_FLAGS if f != "-shared"]
+    jobs = []
+    for src in HIP_SOURCES:
+        obj = os.path.join(objdir, os.path.basename(src) + "." + tag)
+        jobs.append(([HIPCC, *flags, *extra, f"-I{INCLUDE}", f"-I{os.path.join(CSRC, 'hip')}", "-c", src, "-o", obj], obj))
+    with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
+        list(pool.map(lambda j: _run(j[0]), jobs))
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *[j[1] for j in jobs], "-o", out])
+    return out
+
+
 def build_hip(extra=()):
-    srcs = [s for s in HIP_SOURCES if os.path.exists(s)]
-    _run([HIPCC, *HIP_FLAGS, *extra, f"-I{INCLUDE}", f"-I{os.path.join(CSRC, 'hip')}",
-          *srcs, "-o", ATTN_LIB])
-    return ATTN_LIB
+    return _compile_and_link(ATTN_LIB, extra)
 
 
 def build_trace():
-    srcs = [s for s in HIP_SOURCES if os.path.exists(s)]
-    _run([HIPCC, *HIP_FLAGS, "-DMUX_TRACE", f"-I{INCLUDE}", f"-I{os.path.join(CSRC, 'hip')}", *srcs, "-o", TRACE_LIB])
-    return TRACE_LIB
+    return _compile_and_link(TRACE_LIB, ("-DMUX_TRACE",), tag="trace.o")
 
 
 def build_probe():

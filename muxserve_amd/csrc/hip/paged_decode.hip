@@ -99,14 +99,55 @@ struct DecodeParams {
   int32_t partition;
   int32_t last_block;             // num_pool_blocks - 1: table entries are clamped to it
   int32_t n_host_pairs;           // > 0: units come from `pairs`, the device-side context lengths are not read
-  uint2 pairs[kMaxHostPairs];     // x = sequence | partition index << 16, y = clamped context length
+  int32_t rounds;                 // seq_units' R
+  int32_t absorb;                 // seq_units' A
+  uint2 pairs[kMaxHostPairs];     // x = sequence | unit index << 16, y = clamped context length
 };
 static_assert(sizeof(DecodeParams) <= 4096, "kernel argument segment");
 
 // One unit of work, uniform across the workgroup.
 struct Unit {
-  int item, seq, split, ctx, wh, t0, t1;
+  int item, seq, split, ctx, wh, t0, t1, n_splits;
 };
+
+// How a context of c tokens is cut into units.  P = partition: the tokens the
+// waves of a workgroup load in one round (a multiple of 64); R = rounds: the
+// most full groups of P tokens one unit walks; A = absorb.
+//   fg = c / P full groups, rem = c - fg P tokens behind them.  A remainder of
+//   at most A tokens behind at least one full group is left to the unit that
+//   holds the last group (one more, short, round for one of its waves) instead
+//   of becoming a unit of its own.
+//   nb = ceil(fg / R) units share the fg groups as evenly as possible (unit j
+//   holds fg / nb groups, the first fg % nb units one more); a remainder unit,
+//   index nb, follows when rem > 0.
+// A context with a single unit writes its output directly; others go through
+// the partials and the arrival counter.  Host and device enumerate with this one
+// function, so the units - and with them the rounding of the results - do not
+// depend on who enumerated.
+struct SeqUnits {
+  int fg, nb, rem;
+  __host__ __device__ int count() const { return nb + (rem > 0 ? 1 : 0); }
+};
+__host__ __device__ inline SeqUnits seq_units(int c, int P, int R, int A) {
+  SeqUnits s;
+  s.fg = c / P;
+  s.rem = c - s.fg * P;
+  if (s.fg > 0 && s.rem <= A) s.rem = 0;
+  s.nb = (s.fg + R - 1) / R;
+  return s;
+}
+__host__ __device__ inline void unit_range(int c, int P, const SeqUnits &s, int j, int &t0, int &t1) {
+  if (j < s.nb) {
+    const int base = s.fg / s.nb, extra = s.fg - base * s.nb;
+    const int g0 = j * base + (j < extra ? j : extra);
+    const int g1 = g0 + base + (j < extra ? 1 : 0);
+    t0 = g0 * P;
+    t1 = (j == s.nb - 1 && s.rem == 0) ? c : g1 * P;      // an absorbed remainder rides on the last unit
+  } else {
+    t0 = s.fg * P;
+    t1 = c;
+  }
+}
 
 // Device-coherent accesses for data handed between workgroups of one kernel
 // that may run on different XCDs (each XCD has its own L2).
@@ -343,7 +384,7 @@ __device__ __forceinline__ void merge_and_write(const DecodeItemDev &I, const Un
                                                 const float (*xa)[G][kHeadSize], const float (*xm)[G][2],
                                                 int n_active, int lane) {
   constexpr int D = kHeadSize;
-  const bool single = u.ctx <= partition;
+  const bool single = u.n_splits == 1;
   const int hq0 = u.wh * G;
 #pragma unroll 1
   for (int g = 0; g < G; ++g) {
@@ -384,7 +425,7 @@ __device__ __forceinline__ void merge_and_write(const DecodeItemDev &I, const Un
   // wave's partial stores have been acknowledged before the counter is bumped -
   // the explicit vmcnt wait; (2) the combiner's loads issue after its atomic
   // returned - they depend on its value.  The fences only pin the compiler.
-  const int n_splits = (u.ctx + partition - 1) / partition;
+  const int n_splits = u.n_splits;
   int32_t *counter = I.counters + static_cast<int64_t>(u.seq) * (I.Hq / G) + u.wh;
   wait_own_vector_memory();
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -407,7 +448,7 @@ __device__ __forceinline__ void merge_and_write_group(const DecodeItemDev &I, co
                                                       const float (*xa)[G][kHeadSize], const float (*xm)[G][2],
                                                       int *arrival_lds, int n_active, int lane, int wave) {
   constexpr int D = kHeadSize;
-  const bool single = u.ctx <= partition;
+  const bool single = u.n_splits == 1;
   const int hq0 = u.wh * G;
 #pragma unroll 1
   for (int g = wave; g < G; g += n_active) {
@@ -446,7 +487,7 @@ __device__ __forceinline__ void merge_and_write_group(const DecodeItemDev &I, co
   // bypass the per-XCD L2, so the acknowledgement is all that is needed), the
   // workgroup meets, one lane announces the arrival and tells the others
   // whether this workgroup came last.
-  const int n_splits = (u.ctx + partition - 1) / partition;
+  const int n_splits = u.n_splits;
   int32_t *counter = I.counters + static_cast<int64_t>(u.seq) * (I.Hq / G) + u.wh;
   wait_own_vector_memory();
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -467,16 +508,16 @@ __device__ __forceinline__ void merge_and_write_group(const DecodeItemDev &I, co
 // lengths in global memory.
 // ---------------------------------------------------------------------------
 
-// Maps pair index e to (sequence, partition index).  Every lane returns the
-// same answer; false: e is past the last pair (grid padding).  Pairs are
-// numbered in three classes, chosen so that the kernel's last workgroups are
-// the ones that finish fastest:
-//   1. the remainder (ctx % partition tokens) of every sequence longer than one
-//      partition - dispatched first, so the partition that arrives last and
-//      combines a split sequence is normally a full one in mid-kernel;
-//   2. all full partitions of those sequences;
-//   3. sequences that fit one partition (ctx <= partition): no partials, no
-//      atomics, the output is written straight from the workgroup.
+// Maps pair index e to (sequence, unit index).  Every lane returns the same
+// answer; false: e is past the last pair (grid padding).  Pairs are numbered in
+// three classes, chosen so that the kernel's last workgroups are the ones that
+// finish fastest:
+//   1. the remainder unit of every context that has more than one unit -
+//      dispatched first, so the unit that arrives last and combines a split
+//      context is normally a full one in mid-kernel;
+//   2. all other units of those contexts;
+//   3. contexts with a single unit: no partials, no atomics, the output is
+//      written straight from the workgroup.
 
 // Lane index of the n-th (0-based) set bit of a wave mask that has more than n bits set.
 __device__ __forceinline__ int nth_set_lane(unsigned long long mask, int n, int lane) {
@@ -491,23 +532,26 @@ __device__ __forceinline__ int nth_set_lane(unsigned long long mask, int n, int 
 // single memory latency.
 constexpr int kLocateChunks = 4;
 __device__ __forceinline__ bool locate_pair_small(const int32_t *ctx_arr, int B, int max_ctx, int partition,
-                                                  int e, int lane, int &seq, int &split, int &ctx) {
-  int c[kLocateChunks], full[kLocateChunks];
+                                                  int rounds, int absorb, int e, int lane, int &seq, int &split,
+                                                  int &ctx) {
+  int c[kLocateChunks], big[kLocateChunks];
 #pragma unroll
   for (int j = 0; j < kLocateChunks; ++j) {
     const int s = 64 * j + lane;
     c[j] = s < B ? ctx_arr[s] : 0;
   }
-  unsigned long long rem_mask[kLocateChunks];
+  unsigned long long rem_mask[kLocateChunks], single_mask[kLocateChunks];
 #pragma unroll
   for (int j = 0; j < kLocateChunks; ++j) {
     c[j] = max(min(c[j], max_ctx), 0);
-    const int q = c[j] / partition;
-    full[j] = c[j] > partition ? q : 0;
-    rem_mask[j] = __builtin_amdgcn_ballot_w64(c[j] > partition && c[j] != q * partition);
+    const SeqUnits su = seq_units(c[j], partition, rounds, absorb);
+    const bool split_ctx = su.count() > 1;
+    big[j] = split_ctx ? su.nb : 0;
+    rem_mask[j] = __builtin_amdgcn_ballot_w64(split_ctx && su.rem > 0);
+    single_mask[j] = __builtin_amdgcn_ballot_w64(c[j] > 0 && !split_ctx);
   }
   int base = 0;
-  // class 1: remainders of split sequences
+  // class 1: remainder units of split contexts
 #pragma unroll
   for (int j = 0; j < kLocateChunks; ++j) {
     const int cnt = __popcll(rem_mask[j]);
@@ -515,32 +559,31 @@ __device__ __forceinline__ bool locate_pair_small(const int32_t *ctx_arr, int B,
       const int k = nth_set_lane(rem_mask[j], e - base, lane);
       seq = 64 * j + k;
       ctx = __builtin_amdgcn_readlane(c[j], k);
-      split = ctx / partition;
+      split = __builtin_amdgcn_readlane(big[j], k);
       return true;
     }
     base += cnt;
   }
-  // class 2: full partitions of split sequences
+  // class 2: the other units of split contexts
 #pragma unroll
   for (int j = 0; j < kLocateChunks; ++j) {
-    const int incl = wave_inclusive_scan(full[j]);
+    const int incl = wave_inclusive_scan(big[j]);
     const int total = __builtin_amdgcn_readlane(incl, 63);
     if (e < base + total) {
       const int k = __popcll(__builtin_amdgcn_ballot_w64(base + incl <= e));
       seq = 64 * j + k;
-      split = e - base - __builtin_amdgcn_readlane(incl - full[j], k);
+      split = e - base - __builtin_amdgcn_readlane(incl - big[j], k);
       ctx = __builtin_amdgcn_readlane(c[j], k);
       return true;
     }
     base += total;
   }
-  // class 3: sequences that fit one partition
+  // class 3: contexts with a single unit
 #pragma unroll
   for (int j = 0; j < kLocateChunks; ++j) {
-    const unsigned long long mask = __builtin_amdgcn_ballot_w64(c[j] > 0 && c[j] <= partition);
-    const int cnt = __popcll(mask);
+    const int cnt = __popcll(single_mask[j]);
     if (e < base + cnt) {
-      const int k = nth_set_lane(mask, e - base, lane);
+      const int k = nth_set_lane(single_mask[j], e - base, lane);
       seq = 64 * j + k;
       ctx = __builtin_amdgcn_readlane(c[j], k);
       split = 0;
@@ -563,7 +606,8 @@ __device__ __forceinline__ bool locate_pair(const DecodeParams &P, const DecodeI
     ctx = static_cast<int>(pr.y);
     return true;
   }
-  if (I.unit_table == nullptr) return locate_pair_small(I.ctx, I.B, I.max_ctx, partition, e, lane, seq, split, ctx);
+  if (I.unit_table == nullptr)
+    return locate_pair_small(I.ctx, I.B, I.max_ctx, partition, P.rounds, P.absorb, e, lane, seq, split, ctx);
   const int4 ent = I.unit_table[e];
   if (ent.x < 0) return false;
   seq = ent.x;
@@ -572,7 +616,7 @@ __device__ __forceinline__ bool locate_pair(const DecodeParams &P, const DecodeI
   return true;
 }
 
-// Writes the (sequence, partition) table of one item per workgroup, in the same
+// Writes the (sequence, unit) table of one item per workgroup, in the same
 // three classes as above.  Thread t owns a contiguous range of sequences;
 // class counts are prefix-summed over the threads in LDS.  Entries past the
 // last pair (the grid is sized from an upper bound) get sequence -1.
@@ -583,7 +627,7 @@ struct PlanItem {
 };
 struct PlanParams {
   PlanItem it[MUXA_MAX_DECODE_ITEMS];
-  int32_t partition;
+  int32_t partition, rounds, absorb;
 };
 
 __global__ __launch_bounds__(256) void decode_plan_kernel(const PlanParams PP) {
@@ -596,10 +640,10 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(const PlanParams PP) {
   int n[3] = {0, 0, 0};
   for (int s = s0; s < s1; ++s) {
     const int c = max(min(I.ctx[s], I.max_ctx), 0);
-    const int q = c / partition;
-    if (c > partition) {
-      n[1] += q;
-      if (c != q * partition) n[0] += 1;
+    const SeqUnits su = seq_units(c, partition, PP.rounds, PP.absorb);
+    if (su.count() > 1) {
+      n[1] += su.nb;
+      if (su.rem > 0) n[0] += 1;
     } else if (c > 0) {
       n[2] += 1;
     }
@@ -622,11 +666,11 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(const PlanParams PP) {
   int at2 = tot0 + tot1 + scan[2][t] - n[2];
   for (int s = s0; s < s1; ++s) {
     const int c = max(min(I.ctx[s], I.max_ctx), 0);
-    const int q = c / partition;
-    if (c > partition) {
-      for (int j = 0; j < q; ++j)
+    const SeqUnits su = seq_units(c, partition, PP.rounds, PP.absorb);
+    if (su.count() > 1) {
+      for (int j = 0; j < su.nb; ++j)
         if (at1 < I.capacity) I.table[at1++] = make_int4(s, j, c, 0);
-      if (c != q * partition && at0 < I.capacity) I.table[at0++] = make_int4(s, q, c, 0);
+      if (su.rem > 0 && at0 < I.capacity) I.table[at0++] = make_int4(s, su.nb, c, 0);
     } else if (c > 0) {
       if (at2 < I.capacity) I.table[at2++] = make_int4(s, 0, c, 0);
     }
@@ -687,10 +731,13 @@ __global__ MUX_DECODE_BOUNDS void paged_decode_kernel(const DecodeParams P) {
   const int partition = P.partition;
   // Every wave of the workgroup derives the same unit (or all of them leave).
   if (!locate_pair(P, I, partition, e, lane, u.seq, u.split, u.ctx)) return;
-  u.t0 = u.split * partition;
-  u.t1 = min(u.ctx, u.t0 + partition);
+  {
+    const SeqUnits su = seq_units(u.ctx, partition, P.rounds, P.absorb);
+    unit_range(u.ctx, partition, su, u.split, u.t0, u.t1);
+    u.n_splits = su.count();
+  }
   MUX_TR(1);
-  MUX_TRV(7, static_cast<long long>(u.t1 - u.t0) | (static_cast<long long>(u.ctx > partition) << 16));
+  MUX_TRV(7, static_cast<long long>(u.t1 - u.t0) | (static_cast<long long>(u.n_splits > 1) << 16));
   const int hq0 = u.wh * G;
   const int hk = hq0 / I.ratio;
 
@@ -828,8 +875,11 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
   u.wh = local - e * WH;
   const int partition = P.partition;
   if (!locate_pair(P, I, partition, e, lane, u.seq, u.split, u.ctx)) return;
-  u.t0 = u.split * partition;
-  u.t1 = min(u.ctx, u.t0 + partition);
+  {
+    const SeqUnits su = seq_units(u.ctx, partition, P.rounds, P.absorb);
+    unit_range(u.ctx, partition, su, u.split, u.t0, u.t1);
+    u.n_splits = su.count();
+  }
   const int hq0 = u.wh * G;
   const int hk = hq0 / I.ratio;
   const int t1 = u.t1;
@@ -1040,6 +1090,12 @@ namespace {
 
 int pick_group(int ratio);
 
+// EXPERIMENT: policy knobs from the environment.
+int env_int(const char *name, int dflt) {
+  const char *v = getenv(name);
+  return v && *v ? atoi(v) : dflt;
+}
+
 // Tokens per partition when the caller leaves the choice to the library: short
 // partitions spread the batch over more workgroups, long ones amortise a unit's
 // fixed cost; the grouped-query kernel streams a partition with its loads
@@ -1055,6 +1111,14 @@ int choose_partition(const MuxDecodeItem *items, int n_items, int requested) {
   }
   if (max_ctx <= 4096) return 256;
   return all_grouped ? 1024 : 512;
+}
+
+// The other two knobs of seq_units.
+struct DecodePolicy {
+  int rounds, absorb;
+};
+DecodePolicy choose_policy(const MuxDecodeItem *, int, int) {
+  return DecodePolicy{env_int("MUX_DECODE_ROUNDS", 1), env_int("MUX_DECODE_ABSORB", 0)};
 }
 
 int pick_group(int ratio) {
@@ -1120,12 +1184,13 @@ size_t plan_workspace(const MuxDecodeItem *items, int n_items, int partition, It
   return off;
 }
 
-// Host-side enumeration of one item's (sequence, partition) pairs, in the
-// order the device-side enumeration (locate_pair_small) uses: remainders of
-// split sequences, their full partitions, then the sequences that fit one
-// partition.  Appends to out[*n]; false when they do not fit the kernel
-// argument's table or its 16-bit fields.
-bool enumerate_pairs_on_host(const int32_t *ctx_host, int B, int max_ctx, int partition, uint2 *out, int *n) {
+// Host-side enumeration of one item's (sequence, unit) pairs, in the order the
+// device-side enumeration (locate_pair_small) uses: remainder units of split
+// contexts, their other units, then the contexts with a single unit.  Appends
+// to out[*n]; false when they do not fit the kernel argument's table or its
+// 16-bit fields.
+bool enumerate_pairs_on_host(const int32_t *ctx_host, int B, int max_ctx, int partition, int rounds, int absorb,
+                             uint2 *out, int *n) {
   if (B > 0xffff) return false;
   auto clamped = [&](int s) { return std::max(std::min(ctx_host[s], max_ctx), 0); };
   int at = *n;
@@ -1135,18 +1200,20 @@ bool enumerate_pairs_on_host(const int32_t *ctx_host, int B, int max_ctx, int pa
     return true;
   };
   for (int s = 0; s < B; ++s) {
-    const int c = clamped(s), q = c / partition;
-    if (c > partition && c != q * partition && !push(s, q, c)) return false;
+    const int c = clamped(s);
+    const SeqUnits su = seq_units(c, partition, rounds, absorb);
+    if (su.count() > 1 && su.rem > 0 && !push(s, su.nb, c)) return false;
   }
   for (int s = 0; s < B; ++s) {
-    const int c = clamped(s), q = c / partition;
-    if (c > partition)
-      for (int j = 0; j < q; ++j)
+    const int c = clamped(s);
+    const SeqUnits su = seq_units(c, partition, rounds, absorb);
+    if (su.count() > 1)
+      for (int j = 0; j < su.nb; ++j)
         if (!push(s, j, c)) return false;
   }
   for (int s = 0; s < B; ++s) {
     const int c = clamped(s);
-    if (c > 0 && c <= partition && !push(s, 0, c)) return false;
+    if (c > 0 && seq_units(c, partition, rounds, absorb).count() == 1 && !push(s, 0, c)) return false;
   }
   *n = at;
   return true;
@@ -1219,6 +1286,31 @@ size_t mux_paged_decode_workspace_bytes(const MuxDecodeItem *items, int32_t n_it
   return mux::plan_workspace(items, n_items, partition, nullptr);
 }
 
+int32_t mux_paged_decode_host_pairs(const MuxDecodeItem *items, int32_t n_items, int32_t partition_size) {
+  using namespace mux;
+  if (!items || n_items <= 0 || n_items > MUXA_MAX_DECODE_ITEMS) return 0;
+  if (partition_size < 0 || partition_size % 64 != 0) return 0;
+  for (int i = 0; i < n_items; ++i)
+    if (items[i].num_kv_heads <= 0 || items[i].num_q_heads <= 0 || items[i].num_q_heads % items[i].num_kv_heads != 0)
+      return 0;
+  const int partition = choose_partition(items, n_items, partition_size);
+  const DecodePolicy pol = choose_policy(items, n_items, partition);
+  // The first launch group: the items that share the first item's head grouping.
+  const int G = pick_group(items[0].num_q_heads / items[0].num_kv_heads);
+  uint2 pairs[kMaxHostPairs];
+  int n_pairs = 0;
+  for (int i = 0; i < n_items; ++i) {
+    const MuxDecodeItem &it = items[i];
+    if (pick_group(it.num_q_heads / it.num_kv_heads) != G) continue;
+    if (it.num_seqs <= 0 || it.max_context_len <= 0) continue;
+    if (!it.context_lens_host ||
+        !enumerate_pairs_on_host(it.context_lens_host, it.num_seqs, it.max_context_len, partition, pol.rounds,
+                                 pol.absorb, pairs, &n_pairs))
+      return 0;
+  }
+  return n_pairs;
+}
+
 int32_t mux_paged_decode_workspace_init(void *workspace, size_t workspace_bytes, void *stream) {
   if (!workspace || workspace_bytes == 0) return MUXA_OK;
   if (reinterpret_cast<uintptr_t>(workspace) & 15u) return MUXA_EINVAL;
@@ -1255,6 +1347,8 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
     if (rc != MUXA_OK) return rc;
   }
   const int partition = choose_partition(items, n_items, partition_size);
+  const DecodePolicy pol = choose_policy(items, n_items, partition);
+  const int rounds = pol.rounds, absorb = pol.absorb;
   ItemPlan plan[MUXA_MAX_DECODE_ITEMS];
   const size_t need = plan_workspace(items, n_items, partition, plan);
   if (need == SIZE_MAX) return MUXA_EUNSUPPORTED;   // more (sequence, head group) pairs than counters
@@ -1271,10 +1365,14 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
     DecodeParams P = {};
     PlanParams PP;
     PP.partition = partition;
+    PP.rounds = rounds;
+    PP.absorb = absorb;
     int n_tables = 0;
     P.k_pool = k_pool;
     P.v_pool = v_pool;
     P.partition = partition;
+    P.rounds = rounds;
+    P.absorb = absorb;
     P.last_block = static_cast<int32_t>(std::min<int64_t>(num_pool_blocks - 1, 0x7fffffff));
     P.n_items = 0;
     P.n_host_pairs = 0;
@@ -1291,7 +1389,7 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
         pair_begin[i] = n_pairs;
         host_pairs = it.context_lens_host != nullptr &&
                      enumerate_pairs_on_host(it.context_lens_host, it.num_seqs, it.max_context_len, partition,
-                                             P.pairs, &n_pairs);
+                                             rounds, absorb, P.pairs, &n_pairs);
         pair_end[i] = n_pairs;
       }
       host_pairs = host_pairs && n_pairs > 0;
@@ -1458,7 +1556,7 @@ int32_t mux_paged_decode(void *out, int64_t out_row_stride, const void *q, int64
                          int32_t block_size, int32_t max_blocks, int32_t max_context_len,
                          float scale, int32_t dtype, int32_t partition_size,
                          void *workspace, size_t workspace_bytes, void *stream) {
-  MuxDecodeItem it;
+  MuxDecodeItem it = {};     // every field the wrapper does not name (context_lens_host, ...) is null / zero
   it.out = out;
   it.q = q;
   it.out_row_stride = out_row_stride;

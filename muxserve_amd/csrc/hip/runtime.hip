@@ -5,7 +5,7 @@
 
 extern "C" {
 
-int32_t mux_attn_version(void) { return 100; }
+int32_t mux_attn_version(void) { return 300; }
 
 int32_t mux_last_hip_error(void) { return mux::g_last_hip_error; }
 

@@ -188,7 +188,7 @@ MuxDecodeItem decode_item(const at::Tensor &out, const at::Tensor &q, const at::
   TORCH_CHECK(q.dim() == 2 && q.size(1) % kHead == 0 && q.size(0) >= B && out.sizes() == q.sizes() &&
                   q.scalar_type() == out.scalar_type(),
               "q/out: expected [>=B, Hq*128] of equal shape and dtype");
-  MuxDecodeItem it;
+  MuxDecodeItem it = {};
   it.out = out.data_ptr();
   it.q = q.data_ptr();
   it.out_row_stride = rows(out, "out");

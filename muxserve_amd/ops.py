@@ -191,6 +191,50 @@ def multi_decode(calls: List[DecodeCall], k_pool: torch.Tensor, v_pool: torch.Te
     _lib.check_attn(rc, "mux_multi_decode")
 
 
+class DecodeLaunch:
+    """A fused decode launch prepared once and issued many times.
+
+    The serving loop runs the same step shape for every layer of a model, and a
+    benchmark loop repeats the same batch: the tensor checks, the descriptor
+    array and the workspace are made here, once, and ``launch()`` is a single
+    call into the C ABI.  The tensors of `calls` (and the host copies of the
+    context lengths) must stay alive and unchanged in shape while the object is
+    used; their contents may change between launches."""
+
+    def __init__(self, calls: List[DecodeCall], k_pool: torch.Tensor, v_pool: torch.Tensor,
+                 partition_size: int = 0, workspace: Optional[torch.Tensor] = None, stream=None):
+        if not 1 <= len(calls) <= _lib.MUXA_MAX_DECODE_ITEMS:
+            raise ValueError(f"1..{_lib.MUXA_MAX_DECODE_ITEMS} models per launch")
+        _need_cuda(k_pool, v_pool)
+        bs = _check_pools(k_pool, v_pool)
+        for c in calls:
+            if c.q.dtype != k_pool.dtype:
+                raise TypeError("q dtype must equal the pool dtype")
+        self.calls = list(calls)                  # keeps the tensors alive
+        self.pools = (k_pool, v_pool)
+        self.items = (_lib.MuxDecodeItem * len(calls))(*[c.to_item() for c in calls])
+        lib = _lib.attn()
+        need = lib.mux_paged_decode_workspace_bytes(ctypes.addressof(self.items), len(calls), int(partition_size))
+        self.stream_ptr = _stream_ptr(stream)
+        self.workspace = workspace if workspace is not None else _workspace(need, k_pool.device, self.stream_ptr)
+        ws = self.workspace
+        ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel() * ws.element_size()) if ws is not None else (None, 0)
+        # (sequence, unit) pairs enumerated on the host; 0: the units are enumerated on the device
+        self.host_pairs = int(lib.mux_paged_decode_host_pairs(ctypes.addressof(self.items), len(calls),
+                                                              int(partition_size)))
+        self._fn = lib.mux_multi_decode
+        self._args = (ctypes.addressof(self.items), len(calls), k_pool.data_ptr(), v_pool.data_ptr(),
+                      k_pool.shape[0], HEAD_SIZE, bs, _dtype_code(k_pool), int(partition_size), ws_ptr, ws_bytes,
+                      self.stream_ptr)
+
+    def launch(self) -> None:
+        rc = self._fn(*self._args)
+        if rc != 0:
+            _lib.check_attn(rc, "mux_multi_decode")
+
+    __call__ = launch
+
+
 def multi_decode_noalloc(calls: List[DecodeCall], k_pool: torch.Tensor, v_pool: torch.Tensor,
                          partition_size: int = 0, stream=None) -> None:
     """multi_decode through the entry point that allocates nothing: scratch is

@@ -116,3 +116,121 @@ def test_grid_bound_from_the_context_sum_covers_every_pair():
             true_pairs = int((-(-ctx // partition)).sum())
             assert reserved >= true_pairs, (partition, trial, reserved, true_pairs)
             assert reserved <= min(B * max_splits, int(ctx.sum()) // partition + B) + 15
+
+
+# ---------------------------------------------------------------------------
+# Every entry point of include/muxserve_attn.h called once with well-formed
+# arguments.  No device is present where this runs, so nothing can be launched:
+# each call has to come back with a return code - MUXA_EHIP where it got as far
+# as the HIP runtime, MUXA_OK where the host side had nothing to launch, a byte
+# or pair count for the sizing helpers - and never crash the host on the way
+# (an uninitialised field of a descriptor built inside the library once did).
+# "Device" pointers are made-up aligned addresses: the host side must not
+# dereference them.  Host arrays (context_lens_host, prompt_lens_host, the
+# descriptor arrays, output words) are real.
+# ---------------------------------------------------------------------------
+def _call_table():
+    import numpy as np
+    P = lambda k: 0x7F0000000000 + 0x100000 * k          # noqa: E731  fake, 1 MiB apart, 16-byte aligned
+    keep = []
+    ctx_host = np.array([5, 200, 300, 17], dtype=np.int32)
+    keep.append(ctx_host)
+
+    def decode_items(n=1, host=True):
+        arr = (_lib.MuxDecodeItem * n)()
+        for it in arr:
+            it.out, it.q, it.out_row_stride, it.q_row_stride = P(1), P(2), 4 * 128, 4 * 128
+            it.block_tables, it.context_lens = P(3), P(4)
+            it.total_context_len, it.layer, it.num_layers, it.num_seqs = 522, 0, 1, 4
+            it.num_q_heads, it.num_kv_heads, it.max_blocks, it.max_context_len, it.scale = 4, 4, 19, 300, 0.088
+            it.context_lens_host = ctx_host.ctypes.data if host else None
+        keep.append(arr)
+        return ctypes.addressof(arr)
+
+    lens = (ctypes.c_int32 * 2)(40, 9)
+    pit = (_lib.MuxPrefillItem * 1)()
+    pit[0].out, pit[0].out_row_stride, pit[0].q, pit[0].q_row_stride = P(1), 512, P(2), 512
+    pit[0].k, pit[0].v, pit[0].kv_row_stride, pit[0].cu_seqlens = P(3), P(4), 512, P(5)
+    pit[0].prompt_lens_host, pit[0].num_prompts, pit[0].max_prompt_len = ctypes.addressof(lens), 2, 40
+    pit[0].num_q_heads, pit[0].num_kv_heads, pit[0].scale = 4, 4, 0.088
+    cw = (_lib.MuxCacheWriteItem * 1)()
+    cw[0].k, cw[0].v, cw[0].kv_row_stride, cw[0].slot_mapping = P(3), P(4), 512, P(6)
+    cw[0].layer, cw[0].num_layers, cw[0].num_tokens, cw[0].num_kv_heads = 0, 1, 8, 4
+    words = (ctypes.c_uint32 * 8)()
+    info = (ctypes.c_int32 * 2)()
+    sout = ctypes.c_void_p()
+    ncu = ctypes.c_int32()
+    keep += [lens, pit, cw, words, info, sout, ncu]
+    ws = 1 << 22
+    table = {
+        "mux_attn_version": lambda f: f(),
+        "mux_last_hip_error": lambda f: f(),
+        "mux_reshape_and_cache": lambda f: f(P(3), P(4), 512, P(7), P(8), 64, P(6), 0, 1, 8, 4, 128, 16, 0, None),
+        "mux_paged_decode_workspace_bytes": lambda f: f(decode_items(2), 2, 0),
+        "mux_paged_decode_host_pairs": lambda f: f(decode_items(2), 2, 0),
+        "mux_paged_decode_workspace_init": lambda f: f(P(9), ws, None),
+        "mux_multi_decode": lambda f: f(decode_items(2), 2, P(7), P(8), 64, 128, 16, 0, 0, P(9), ws, None),
+        "mux_multi_decode_noalloc_max_bytes": lambda f: f(),
+        "mux_multi_decode_noalloc": lambda f: f(decode_items(2, host=False), 2, P(7), P(8), 64, 128, 16, 0, 0, None),
+        "mux_paged_decode": lambda f: f(P(1), 512, P(2), 512, P(7), P(8), 64, P(3), P(4), 0, 1, 4, 4, 4, 128, 16, 19,
+                                        300, 0.088, 0, 0, P(9), ws, None),
+        "mux_prefill_causal": lambda f: f(P(1), 512, P(2), 512, P(3), P(4), 512, P(5), None, ctypes.addressof(lens), 2,
+                                          40, 4, 4, 128, 0.088, 0, None),
+        "mux_multi_prefill_causal": lambda f: f(ctypes.addressof(pit), 1, 128, 0, None),
+        "mux_rotary_neox": lambda f: f(P(5), P(2), 512, P(3), 512, P(6), 4096, 128, 8, 4, 4, 128, 0, None),
+        "mux_rope_reshape_and_cache": lambda f: f(P(5), P(2), 512, P(3), P(4), 512, P(6), 4096, 128, P(7), P(8), 64,
+                                                  P(10), 0, 1, 8, 4, 4, 128, 16, 0, None),
+        "mux_multi_rope_reshape_and_cache": lambda f: f(ctypes.addressof(cw), 1, P(7), P(8), 64, 128, 16, 0, None),
+        "mux_rms_norm": lambda f: f(P(1), 4096, P(2), 4096, P(3), 1e-6, 8, 4096, 0, None),
+        "mux_silu_and_mul": lambda f: f(P(1), 1024, P(2), 2048, 8, 1024, 0, None),
+        "mux_greedy_sample_workspace_bytes": lambda f: f(32000),
+        "mux_greedy_sample_workspace_init": lambda f: f(P(9), ws, None),
+        "mux_greedy_sample": lambda f: f(P(1), P(2), 4096, 8, None, 8, P(3), 4096, 32000, 32000, 4096, 0, P(9), ws,
+                                         None),
+        "mux_build_step_inputs": lambda f: f(P(1), 8, 16, 2, 4, 16, P(2), 4, P(3), 40, 1, 4, P(4), P(5), 16, None),
+        "mux_cu_parts_mask": lambda f: f(0b1001, 256, ctypes.addressof(words), 8),
+        "mux_stream_create_cu_parts": lambda f: f(ctypes.byref(sout), 0b11, ctypes.byref(ncu)),
+        "mux_stream_create_cu_range": lambda f: f(ctypes.byref(sout), 0, 40, ctypes.byref(ncu)),
+        "mux_stream_destroy": lambda f: f(None),
+        "mux_device_cu_info": lambda f: f(ctypes.addressof(info)),
+    }
+    return table, keep
+
+
+def test_every_attn_entry_point_returns_a_code_when_called_without_a_device():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a device is present: the made-up device pointers of this test must not reach a kernel")
+    lib = _lib.attn()
+    table, keep = _call_table()
+    assert set(table) == set(_declared("muxserve_attn.h")), sorted(set(table) ^ set(_declared("muxserve_attn.h")))
+    sizes = {"mux_paged_decode_workspace_bytes", "mux_multi_decode_noalloc_max_bytes",
+             "mux_greedy_sample_workspace_bytes"}
+    got = {}
+    for name, call in table.items():
+        got[name] = call(getattr(lib, name))
+    assert got["mux_attn_version"] >= 300
+    assert got["mux_paged_decode_host_pairs"] == 2 * 5          # per item: 300 -> 256 + 44, plus 5, 200, 17
+    assert got["mux_cu_parts_mask"] > 0
+    for name in sizes:
+        assert got[name] > 0, name
+    launches = set(table) - sizes - {"mux_attn_version", "mux_last_hip_error", "mux_paged_decode_host_pairs",
+                                     "mux_cu_parts_mask", "mux_stream_destroy"}
+    for name in sorted(launches):
+        assert got[name] == -4, f"{name} returned {got[name]}, expected MUXA_EHIP (no device)"
+    assert lib.mux_last_hip_error() != 0
+    del keep
+
+
+def test_single_model_decode_wrapper_equals_the_fused_entry_point_on_its_arguments():
+    """mux_paged_decode is mux_multi_decode on one descriptor whose optional
+    fields are absent: both must reject and accept the same calls."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("made-up device pointers")
+    lib = _lib.attn()
+    P = 0x7F0000000000
+    for max_ctx, max_blocks, want in ((300, 19, -4), (300, 18, -1), (0, 0, 0)):
+        rc = lib.mux_paged_decode(P, 512, P + 4096, 512, P + 8192, P + 16384, 64, P + 32768, P + 65536, 0, 1, 4, 4, 4,
+                                  128, 16, max_blocks, max_ctx, 0.088, 0, 0, P + (1 << 20), 1 << 22, None)
+        assert rc == want, (max_ctx, max_blocks, rc)

@@ -497,11 +497,52 @@ def test_decode_config2_full_size_pool(full_size_pool_memory):
     for _ in range(3):
         ops.multi_decode(calls, dk, dv)
     torch.cuda.synchronize()
+    device_enumerated = [m.out.clone() for m in models]
+    # The path the benchmark times: the launch prepared once, the units enumerated on the host
+    # from the host copy of the context lengths.  Same units, so the same bits.
+    host_calls = [ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                                 total_context_len=int(m.context_lens.sum()),
+                                 context_lens_host=torch.from_numpy(np.ascontiguousarray(m.context_lens, dtype=np.int32)))
+                  for m in models]
+    launch = ops.DecodeLaunch(host_calls, dk, dv)
+    assert launch.host_pairs > 0, "the headline batch must take the host-enumerated path"
+    for m in models:
+        m.out.fill_(7.0)
+    for _ in range(3):
+        launch()
+    torch.cuda.synchronize()
+    for m, dev_out in zip(models, device_enumerated):
+        assert torch.equal(m.out[:m.batch], dev_out[:m.batch]), "host- and device-enumerated launches must agree bitwise"
     ks, vs, tables = workloads.compact_to_host(dk, dv, models, bs)
     del dk, dv
     for m, t in zip(models, tables):
         want = orc.paged_decode(m.q.cpu(), ks, vs, t, m.context_lens, m.scale)
         _check(m.out[:m.batch].float().cpu(), want)
+
+
+@pytest.mark.parametrize("n_pairs", [384, 385])
+def test_decode_at_the_limit_of_host_enumerated_pairs(n_pairs):
+    """The kernel argument holds 384 (sequence, unit) pairs.  A batch with
+    exactly that many is enumerated on the host, one with a pair more on the
+    device; both give the device-enumerated result bit for bit and match the
+    oracle."""
+    from muxserve_amd import _lib
+    _announce(f"decode with {n_pairs} pairs")
+    # 128 sequences of three units (two full partitions and a remainder) are 384 pairs
+    ctx = [2 * 256 + 1 + (7 * i) % 200 for i in range(128)]
+    if n_pairs == 385:
+        ctx.append(33)
+    dev_got, want = _decode_case(41, ctx, 1, 1, 16, partition=256)
+    host_got, _ = _decode_case(41, ctx, 1, 1, 16, partition=256, host_lens=True)
+    assert torch.equal(host_got, dev_got)
+    _check(host_got, want)
+    it = _lib.MuxDecodeItem()
+    h = np.asarray(ctx, dtype=np.int32)
+    it.num_seqs, it.num_q_heads, it.num_kv_heads, it.num_layers = len(ctx), 1, 1, 1
+    it.max_context_len, it.max_blocks, it.context_lens_host = int(h.max()), 64, h.ctypes.data
+    import ctypes
+    pairs = _lib.attn().mux_paged_decode_host_pairs(ctypes.addressof(it), 1, 256)
+    assert pairs == (384 if n_pairs == 384 else 0)
 
 
 @pytest.mark.parametrize("Hq,Hkv,dtype", [(4, 4, torch.float16), (16, 2, torch.bfloat16)])

@@ -186,6 +186,19 @@ def test_long_context_gqa_bf16_full_size_pool(full_size_pool_memory):
                          m.scale, total_context_len=int(m.context_lens.sum()))
     torch.cuda.synchronize()
     assert torch.isfinite(m.out[:m.batch].float()).all()
+    # The same launch with the units enumerated on the host (the prepared-launch path): same bits.
+    device_enumerated = m.out.clone()
+    launch = ops.DecodeLaunch([ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                                              total_context_len=int(m.context_lens.sum()),
+                                              context_lens_host=torch.from_numpy(
+                                                  np.ascontiguousarray(m.context_lens, dtype=np.int32)))],
+                              k_pool, v_pool)
+    assert launch.host_pairs > 0
+    m.out.fill_(7.0)
+    for _ in range(2):
+        launch()
+    torch.cuda.synchronize()
+    assert torch.equal(m.out[:m.batch], device_enumerated[:m.batch])
     pick = [0, 17, int(np.argmax(m.context_lens)), int(np.argmin(m.context_lens))]
     sub = workloads.DecodeModel(m.name, m.num_q_heads, m.num_kv_heads, m.context_lens[pick].copy(),
                                 m.block_tables[:, pick].copy(), m.scale)
