@@ -329,10 +329,13 @@ def bench_colocated(args):
     pflops = 4.0 * 52 * D * 4 * (1024 * 1025 / 2)
     s_pre, s_dec = ops.CUMaskedStream(0, 40), ops.CUMaskedStream(40, 100)
 
+    host_lens = [torch.from_numpy(np.ascontiguousarray(m.context_lens, dtype=np.int32)) for m in dsets]
+
     def decode(i, stream=None):
         m = dsets[i % len(dsets)]
         ops.paged_decode(m.out, m.q, k_pool, v_pool, m.d_block_tables, m.d_context_lens, m.max_context_len,
-                         m.scale, total_context_len=int(m.context_lens.sum()), stream=stream)
+                         m.scale, total_context_len=int(m.context_lens.sum()), stream=stream,
+                         context_lens_host=host_lens[i % len(dsets)])
 
     def prefill(i, stream=None):
         ops.prefill_causal(pout, q, k, v, cu, 1024, D ** -0.5, 52, stream=stream)
@@ -491,10 +494,14 @@ def bench_gqa_long(args):
         m = workloads.config5(seed=args.seed + i, num_pool_blocks=N)[0][0].to_device(dev, torch.bfloat16, seed=i)
         sets.append(m)
 
+    launches = [ops.DecodeLaunch([ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                                                 total_context_len=int(m.context_lens.sum()),
+                                                 context_lens_host=None if args.no_host_lens else torch.from_numpy(
+                                                     np.ascontiguousarray(m.context_lens, dtype=np.int32)))],
+                                 k_pool, v_pool, args.partition) for m in sets]
+
     def step(i):
-        m = sets[i % len(sets)]
-        ops.paged_decode(m.out, m.q, k_pool, v_pool, m.d_block_tables, m.d_context_lens, m.max_context_len,
-                         m.scale, partition_size=args.partition, total_context_len=int(m.context_lens.sum()))
+        launches[i % len(launches)]()
 
     ms = _time(step, args.steps, args.warmup)
     nbytes = float(np.mean([workloads.decode_bytes(m.context_lens, 64, 8, bs) for m in sets]))
@@ -505,7 +512,8 @@ def bench_gqa_long(args):
     probe_ms = _time(lambda i: workloads.probe_gather_read(k_pool, v_pool, used[i % len(used)], sink), args.steps, args.warmup)
     probe_bytes = float(np.mean([u.numel() * 8192 for u in used]))
     cfg = {"workload": "gqa_long", "shape": "Hq64/Hkv8, B=64, ctx U[2048,8192], bf16", "pool_gb": round(N * 8192 / 1e9, 1),
-           "bytes_per_step": int(nbytes), "partition": args.partition}
+           "bytes_per_step": int(nbytes), "partition": args.partition,
+           "units_enumerated_on_the_host": [l.host_pairs for l in launches]}
     roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
             "traffic": nbytes * GQA_LONG_TRAFFIC_RATIO,
             "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "

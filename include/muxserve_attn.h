@@ -94,14 +94,13 @@ int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t kv_row_strid
  * the grid, device values above it are clamped.
  * total_context_len: optional host-side upper bound on the sum of
  * context_lens (the serving loop has them on the host before the copy,
- * llm_runtime.py:311-326); it only tightens the grid, 0 = unknown.  It MUST be
- * an upper bound: the grid is sized from it, units are enumerated remainders
- * first, full partitions next, single-partition sequences last, and units
- * beyond the grid are not run - an understated sum first leaves outputs of
- * single-partition sequences unwritten and, beyond those, leaves arrival
- * counters of split sequences non-zero, after which the workspace has to be
- * re-initialised (mux_paged_decode_workspace_init) before its next use.  With
- * context_lens_host the enumeration is exact and this field is not used.
+ * llm_runtime.py:311-326); it only tightens the grid of a launch whose units
+ * are enumerated on the device, 0 = unknown.  A bound that turns out too small
+ * costs time, not results: the units it leaves without a workgroup of their own
+ * are run, one after the other, by the workgroups of the last unit that has
+ * one, so every output is still written and the workspace's arrival counters
+ * still return to zero.  With context_lens_host the enumeration is exact and
+ * this field is not used.
  * context_lens_host: optional HOST copy of context_lens [num_seqs] (same
  * place in the serving loop, llm_runtime.py:311-326: the lengths are a host
  * list before they become a tensor).  When every model of a launch comes with
@@ -115,8 +114,9 @@ int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t kv_row_strid
  * partition_size: tokens per split of a context (multiple of 64), 0 = choose.
  * workspace: scratch for the partial results of split contexts and, for
  * batches of more than 256 sequences, the table that maps workgroups to
- * (sequence, partition) pairs (written by a small kernel launched ahead of
- * the attention kernel on the same stream); at least
+ * (sequence, unit) pairs (written by a small kernel launched ahead of
+ * the attention kernel on the same stream; a row for every pair the shapes
+ * allow, num_seqs * ceil(max_context_len / partition)); at least
  * mux_paged_decode_workspace_bytes(...) bytes, 16-byte aligned; may be NULL
  * when that is 0.  Its first MUXA_DECODE_COUNTER_BYTES bytes are arrival
  * counters that must be ZERO when a launch begins: zero them once with

@@ -80,7 +80,9 @@ struct DecodeItemDev {
   int32_t B, Hq, Hkv, ratio;      // ratio = Hq / Hkv
   int32_t max_blocks, max_splits, max_ctx;
   int32_t work_begin;             // first block of this item in the grid
-  int32_t pair_begin;             // first entry of this item in DecodeParams::pairs (host-enumerated launches)
+  int32_t pair_begin;             // host-enumerated launches: first entry of this item in DecodeParams::pairs;
+                                  // device-enumerated: how many of the item's pairs have a workgroup per head group of
+                                  // their own (the grid is sized from the caller's bound on the sum of the context lengths)
   float scale_log2;               // scale * log2(e)
 };
 
@@ -450,8 +452,10 @@ __device__ __forceinline__ void merge_and_write_group(const DecodeItemDev &I, co
   constexpr int D = kHeadSize;
   const bool single = u.n_splits == 1;
   const int hq0 = u.wh * G;
+  // (a wave that had no tokens but stayed - see the kernels' sweep - only keeps the barriers company)
+  const int g_first = wave < n_active ? wave : G;
 #pragma unroll 1
-  for (int g = wave; g < G; g += n_active) {
+  for (int g = g_first; g < G; g += n_active) {
     // Waves without tokens have left early and wrote nothing.
     float M = xm[0][g][0];
 #pragma unroll
@@ -498,7 +502,7 @@ __device__ __forceinline__ void merge_and_write_group(const DecodeItemDev &I, co
   if (*arrival_lds != n_splits - 1) return;
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 #pragma unroll 1
-  for (int g = wave; g < G; g += n_active) combine_head<T>(I, u.seq, hq0 + g, n_splits, lane);
+  for (int g = g_first; g < G; g += n_active) combine_head<T>(I, u.seq, hq0 + g, n_splits, lane);
   // Ready for the next launch.
   if (wave == 0 && lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -608,6 +612,7 @@ __device__ __forceinline__ bool locate_pair(const DecodeParams &P, const DecodeI
   }
   if (I.unit_table == nullptr)
     return locate_pair_small(I.ctx, I.B, I.max_ctx, partition, P.rounds, P.absorb, e, lane, seq, split, ctx);
+  if (e >= I.B * I.max_splits) return false;      // the table holds a row for every pair there can be
   const int4 ent = I.unit_table[e];
   if (ent.x < 0) return false;
   seq = ent.x;
@@ -704,33 +709,28 @@ __device__ __forceinline__ void fetch_q(const DecodeItemDev &I, int seq, int hq0
 #else
 #define MUX_DECODE_BOUNDS __launch_bounds__(64 * NW)
 #endif
-template <typename T, int BS, int G, int NW>
-__global__ MUX_DECODE_BOUNDS void paged_decode_kernel(const DecodeParams P) {
+
+// LDS of one workgroup of the vector-ALU kernel.
+template <int G, int NW>
+struct DecodeSmem {
+  __attribute__((aligned(16))) float p[NW][G][64];      // per-wave probabilities of a tile
+  __attribute__((aligned(16))) uint32_t q[NW][G][64];   // G > 1: per-wave copy of the group's q
+  float x_acc[NW][G][kHeadSize];                        // per-wave partial outputs
+  float x_ml[NW][G][2];
+};
+
+// One unit, start to finish, by the workgroup's NW waves.  STAY = false: waves
+// that have nothing (more) to do return from the kernel (the function's result
+// tells the caller to return); STAY = true, for a workgroup that goes on to
+// another unit: every wave comes back, after a barrier that makes the LDS
+// partials reusable.
+template <typename T, int BS, int G, int NW, bool STAY>
+__device__ __forceinline__ bool decode_unit(const DecodeParams &P, const DecodeItemDev &I, Unit &u, int e,
+                                            DecodeSmem<G, NW> &sm, int lane, int wave) {
   using Geo = Geometry<BS>;
-  __shared__ __attribute__((aligned(16))) float p_lds[NW][G][64];     // per-wave probabilities of a tile
-  __shared__ __attribute__((aligned(16))) uint32_t q_lds[NW][G][64];  // G > 1: per-wave copy of the group's q
-  __shared__ float x_acc[NW][G][kHeadSize];                           // per-wave partial outputs
-  __shared__ float x_ml[NW][G][2];
-
-  MUX_TR(0);
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int w = blockIdx.x;
-  int ii = 0;
-#pragma unroll
-  for (int k = 1; k < MUXA_MAX_DECODE_ITEMS; ++k)
-    if (k < P.n_items && w >= P.it[k].work_begin) ii = k;
-  const DecodeItemDev I = P.it[ii];       // by value: one round of scalar loads for every field
-
-  const int WH = I.Hq / G;                   // head groups per sequence
-  const int local = w - I.work_begin;
-  const int e = local / WH;
-  Unit u;
-  u.item = ii;
-  u.wh = local - e * WH;
   const int partition = P.partition;
   // Every wave of the workgroup derives the same unit (or all of them leave).
-  if (!locate_pair(P, I, partition, e, lane, u.seq, u.split, u.ctx)) return;
+  if (!locate_pair(P, I, partition, e, lane, u.seq, u.split, u.ctx)) return false;
   {
     const SeqUnits su = seq_units(u.ctx, partition, P.rounds, P.absorb);
     unit_range(u.ctx, partition, su, u.split, u.t0, u.t1);
@@ -749,37 +749,92 @@ __global__ MUX_DECODE_BOUNDS void paged_decode_kernel(const DecodeParams P) {
   const int tb0 = u.t0 + wave * 64;
   // A wave without tokens leaves at once and frees its registers for the next
   // workgroup; the barrier below counts only the waves that are still there.
-  if (tb0 >= u.t1) return;
+  const bool idle = tb0 >= u.t1;
+  if constexpr (!STAY) {
+    if (idle) return false;
+  }
   const int n_active = min(NW, (u.t1 - u.t0 + 63) / 64);
-  int id_next = load_block_id<BS>(trow, tb0, u.t1, lane, P.last_block);
-  uint32_t q_s[64];
-  fetch_q<G>(I, u.seq, hq0, lane, q_s, q_lds[wave]);
-  MUX_TR(2);
+  if (!STAY || !idle) {
+    int id_next = load_block_id<BS>(trow, tb0, u.t1, lane, P.last_block);
+    uint32_t q_s[64];
+    fetch_q<G>(I, u.seq, hq0, lane, q_s, sm.q[wave]);
+    MUX_TR(2);
 
-  float m[G], l[G], acc[G][Geo::VI];
+    float m[G], l[G], acc[G][Geo::VI];
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    m[g] = -INFINITY;
-    l[g] = 0.f;
+    for (int g = 0; g < G; ++g) {
+      m[g] = -INFINITY;
+      l[g] = 0.f;
 #pragma unroll
-    for (int j = 0; j < Geo::VI; ++j) acc[g][j] = 0.f;
+      for (int j = 0; j < Geo::VI; ++j) acc[g][j] = 0.f;
+    }
+    for (int tb = tb0; tb < u.t1; tb += 64 * NW) {
+      const int id = id_next;
+      if (tb + 64 * NW < u.t1) id_next = load_block_id<BS>(trow, tb + 64 * NW, u.t1, lane, P.last_block);
+      uint4 kreg[16];
+      uint4 vreg[Geo::BPT][Geo::VI];
+      issue_tile_loads<BS>(kreg, vreg, kpool, vpool, id, tb, u.t1, lane);
+      MUX_TR(3);
+      consume_tile<T, BS, G>(kreg, vreg, q_s, sm.q[wave], sm.p[wave], m, l, acc, I.scale_log2, tb, u.t1, lane);
+      MUX_TR(4);
+    }
+    stash_wave_partial<BS, G>(m, l, acc, sm.x_acc[wave], sm.x_ml[wave], lane);
   }
-  for (int tb = tb0; tb < u.t1; tb += 64 * NW) {
-    const int id = id_next;
-    if (tb + 64 * NW < u.t1) id_next = load_block_id<BS>(trow, tb + 64 * NW, u.t1, lane, P.last_block);
-    uint4 kreg[16];
-    uint4 vreg[Geo::BPT][Geo::VI];
-    issue_tile_loads<BS>(kreg, vreg, kpool, vpool, id, tb, u.t1, lane);
-    MUX_TR(3);
-    consume_tile<T, BS, G>(kreg, vreg, q_s, q_lds[wave], p_lds[wave], m, l, acc, I.scale_log2, tb, u.t1, lane);
-    MUX_TR(4);
-  }
-  stash_wave_partial<BS, G>(m, l, acc, x_acc[wave], x_ml[wave], lane);
   __syncthreads();
   MUX_TR(5);
-  if (wave != 0) return;
-  merge_and_write<T, G, NW>(I, u, partition, x_acc, x_ml, n_active, lane);
+  if constexpr (!STAY) {
+    if (wave != 0) return false;
+  }
+  if (wave == 0) merge_and_write<T, G, NW>(I, u, partition, sm.x_acc, sm.x_ml, n_active, lane);
   MUX_TR(6);
+  if constexpr (STAY) __syncthreads();
+  return true;
+}
+
+template <typename T, int BS, int G, int NW>
+__global__ MUX_DECODE_BOUNDS void paged_decode_kernel(const DecodeParams P) {
+  __shared__ DecodeSmem<G, NW> sm;
+  MUX_TR(0);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int w = blockIdx.x;
+  int ii = 0;
+#pragma unroll
+  for (int k = 1; k < MUXA_MAX_DECODE_ITEMS; ++k)
+    if (k < P.n_items && w >= P.it[k].work_begin) ii = k;
+  const DecodeItemDev I = P.it[ii];       // by value: one round of scalar loads for every field
+
+  const int WH = I.Hq / G;                   // head groups per sequence
+  const int local = w - I.work_begin;
+  const int e = local / WH;
+  Unit u;
+  u.item = ii;
+  u.wh = local - e * WH;
+  decode_unit<T, BS, G, NW, false>(P, I, u, e, sm, lane, wave);
+}
+
+// A device-enumerated launch is sized from the caller's bound on the sum of the
+// context lengths.  Should that bound have been too small, some (sequence, unit)
+// pairs have no workgroup in the grid above; this kernel, launched behind it
+// with one workgroup per item and head group, runs them one after the other
+// (slow, but every output is written and every arrival counter returns to zero).
+// With a bound that holds its workgroups find nothing and leave.
+template <typename T, int BS, int G, int NW>
+__global__ __launch_bounds__(64 * NW) void paged_decode_sweep_kernel(const DecodeParams P) {
+  __shared__ DecodeSmem<G, NW> sm;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int w = blockIdx.x;
+  int ii = 0;
+#pragma unroll
+  for (int k = 1; k < MUXA_MAX_DECODE_ITEMS; ++k)
+    if (k < P.n_items && w >= P.it[k].work_begin) ii = k;
+  const DecodeItemDev I = P.it[ii];
+  Unit u;
+  u.item = ii;
+  u.wh = w - I.work_begin;                   // one workgroup per head group; work_begin counts those
+  for (int e = I.pair_begin;; ++e)           // pair_begin: the pairs that had a place in the grid above
+    if (!decode_unit<T, BS, G, NW, true>(P, I, u, e, sm, lane, wave)) return;
 }
 
 // ---------------------------------------------------------------------------
@@ -846,35 +901,29 @@ struct GqaTile {
   u32x4_t v[8];
 };
 
-template <typename T, int BS, int G, int NW>
-__global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const DecodeParams P) {
+// LDS of one workgroup of the grouped-query kernel.
+template <typename T, int G, int NW>
+struct GqaSmem {
+  static constexpr int kParts = __is_same(T, BF16) ? 2 : 1;    // bf16 keeps 8 bits of a probability: P as hi + lo parts
+  __attribute__((aligned(16))) uint16_t p[NW][kParts][16][kPRow];
+  __attribute__((aligned(16))) float x_acc[NW][G][kHeadSize];
+  float x_ml[NW][G][2];
+  int arrival;
+};
+
+// One unit by the workgroup's NW waves; STAY as in decode_unit above.
+template <typename T, int BS, int G, int NW, bool STAY>
+__device__ __forceinline__ bool decode_unit_gqa(const DecodeParams &P, const DecodeItemDev &I, Unit &u, int e,
+                                                GqaSmem<T, G, NW> &sm, int lane, int wave) {
   using Geo = Geometry<BS>;
   static_assert(G >= 2 && G <= 16, "group size");
-  // bf16 keeps 8 bits of a probability; P is carried as hi + lo parts then.
-  constexpr int kParts = __is_same(T, BF16) ? 2 : 1;
+  constexpr int kParts = GqaSmem<T, G, NW>::kParts;
   constexpr int kStep = kGqaTile * NW;   // wave w takes tokens t0 + 32 w + kStep n .. +31
-  __shared__ __attribute__((aligned(16))) uint16_t p_lds[NW][kParts][16][kPRow];
-  __shared__ __attribute__((aligned(16))) float x_acc[NW][G][kHeadSize];
-  __shared__ float x_ml[NW][G][2];
-  __shared__ int arrival;
-
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int w = blockIdx.x;
-  int ii = 0;
-#pragma unroll
-  for (int k = 1; k < MUXA_MAX_DECODE_ITEMS; ++k)
-    if (k < P.n_items && w >= P.it[k].work_begin) ii = k;
-  const DecodeItemDev I = P.it[ii];       // by value: one round of scalar loads for every field
-
-  const int WH = I.Hq / G;
-  const int local = w - I.work_begin;
-  const int e = local / WH;
-  Unit u;
-  u.item = ii;
-  u.wh = local - e * WH;
+  auto &p_lds = sm.p;
+  auto &x_acc = sm.x_acc;
+  auto &x_ml = sm.x_ml;
   const int partition = P.partition;
-  if (!locate_pair(P, I, partition, e, lane, u.seq, u.split, u.ctx)) return;
+  if (!locate_pair(P, I, partition, e, lane, u.seq, u.split, u.ctx)) return false;
   {
     const SeqUnits su = seq_units(u.ctx, partition, P.rounds, P.absorb);
     unit_range(u.ctx, partition, su, u.split, u.t0, u.t1);
@@ -885,7 +934,10 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
   const int t1 = u.t1;
 
   // A wave without tokens leaves at once (see the kernel above).
-  if (u.t0 + kGqaTile * wave >= t1) return;
+  const bool idle = u.t0 + kGqaTile * wave >= t1;
+  if constexpr (!STAY) {
+    if (idle) return false;
+  }
   const int n_active = min(NW, (t1 - u.t0 + kGqaTile - 1) / kGqaTile);
 
   const int h = lane & 15;               // this lane's head (columns >= G are padding)
@@ -1062,7 +1114,7 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
 
   // ---- this wave's partial to LDS, in the layout the merge expects ----------------------
   l = sum_with_lane_xor32(sum_with_lane_xor16(l));
-  if (h < G) {
+  if (h < G && !idle) {
 #pragma unroll
     for (int nb = 0; nb < 8; ++nb)
       *reinterpret_cast<float4 *>(&x_acc[wave][h][16 * nb + 4 * g]) =
@@ -1073,8 +1125,51 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
     }
   }
   __syncthreads();
-  merge_and_write_group<T, G, NW>(I, u, partition, x_acc, x_ml, &arrival, n_active, lane, wave);
+  merge_and_write_group<T, G, NW>(I, u, partition, x_acc, x_ml, &sm.arrival, n_active, lane, wave);
+  if constexpr (STAY) __syncthreads();      // the partials in LDS are reused by the next unit
+  return true;
 }
+
+template <typename T, int BS, int G, int NW>
+__global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const DecodeParams P) {
+  __shared__ GqaSmem<T, G, NW> sm;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int w = blockIdx.x;
+  int ii = 0;
+#pragma unroll
+  for (int k = 1; k < MUXA_MAX_DECODE_ITEMS; ++k)
+    if (k < P.n_items && w >= P.it[k].work_begin) ii = k;
+  const DecodeItemDev I = P.it[ii];       // by value: one round of scalar loads for every field
+  const int WH = I.Hq / G;
+  const int local = w - I.work_begin;
+  const int e = local / WH;
+  Unit u;
+  u.item = ii;
+  u.wh = local - e * WH;
+  decode_unit_gqa<T, BS, G, NW, false>(P, I, u, e, sm, lane, wave);
+}
+
+// (pairs that got no place in the grid: see paged_decode_sweep_kernel)
+template <typename T, int BS, int G, int NW>
+__global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_sweep_kernel(const DecodeParams P) {
+  __shared__ GqaSmem<T, G, NW> sm;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int w = blockIdx.x;
+  int ii = 0;
+#pragma unroll
+  for (int k = 1; k < MUXA_MAX_DECODE_ITEMS; ++k)
+    if (k < P.n_items && w >= P.it[k].work_begin) ii = k;
+  const DecodeItemDev I = P.it[ii];
+  Unit u;
+  u.item = ii;
+  u.wh = w - I.work_begin;
+  for (int e = I.pair_begin;; ++e)
+    if (!decode_unit_gqa<T, BS, G, NW, true>(P, I, u, e, sm, lane, wave)) return;
+}
+
+
 
 // Zero-fills the arrival counters (a kernel rather than a memset node so the
 // call can be captured into a graph).
@@ -1089,12 +1184,6 @@ __global__ void fill_zero_kernel(int32_t *p, int64_t n) {
 namespace {
 
 int pick_group(int ratio);
-
-// EXPERIMENT: policy knobs from the environment.
-int env_int(const char *name, int dflt) {
-  const char *v = getenv(name);
-  return v && *v ? atoi(v) : dflt;
-}
 
 // Tokens per partition when the caller leaves the choice to the library: short
 // partitions spread the batch over more workgroups, long ones amortise a unit's
@@ -1113,13 +1202,17 @@ int choose_partition(const MuxDecodeItem *items, int n_items, int requested) {
   return all_grouped ? 1024 : 512;
 }
 
-// The other two knobs of seq_units.
+// The other two knobs of seq_units.  Measured on the mixed three-model batch
+// (interleaved runs in one process, medians of eight): units of two to four
+// groups per workgroup 79 - 80 us against 74.5 with one (a wave's second round
+// starts with nothing in flight); a remainder of at most 8 / 16 / 24 tokens left
+// to the last unit 73.6 - 73.7 us against 74.1 - 74.5 without (32: 74.4, 64:
+// 74.7): a remainder of one pool block is cheaper as one more short round of one
+// wave than as a workgroup of its own with its own partial and hand-off.
 struct DecodePolicy {
   int rounds, absorb;
 };
-DecodePolicy choose_policy(const MuxDecodeItem *, int, int) {
-  return DecodePolicy{env_int("MUX_DECODE_ROUNDS", 1), env_int("MUX_DECODE_ABSORB", 0)};
-}
+DecodePolicy choose_policy(const MuxDecodeItem *, int, int) { return DecodePolicy{1, 16}; }
 
 int pick_group(int ratio) {
   if (ratio == 8 || ratio == 4 || ratio == 2) return ratio;
@@ -1133,7 +1226,7 @@ int pick_group(int ratio) {
 struct ItemPlan {
   size_t counters_off, acc_off, ml_off;
   int max_splits;
-  int64_t units;      // (sequence, partition) pairs reserved in the direct kernel's grid
+  int64_t units;      // (sequence, unit) pairs that get a place in the grid of a device-enumerated launch
   size_t table_off;   // pair table of a large batch (0: none)
 };
 
@@ -1172,9 +1265,12 @@ size_t plan_workspace(const MuxDecodeItem *items, int n_items, int partition, It
       off = (off + 255) & ~static_cast<size_t>(255);
     }
     if (it.num_seqs > 64 * kLocateChunks && it.max_context_len > 0) {
+      // A row for every pair there can be, whatever the caller's bound on the sum
+      // says: the bound only sizes the grid, and pairs it leaves without a place
+      // are still found in the table (by the sweep of the kernels).
       any = true;
       w.table_off = off;
-      off += static_cast<size_t>(w.units) * sizeof(int4);
+      off += static_cast<size_t>(it.num_seqs) * w.max_splits * sizeof(int4);
       off = (off + 255) & ~static_cast<size_t>(255);
     }
     if (out) out[i] = w;
@@ -1184,7 +1280,7 @@ size_t plan_workspace(const MuxDecodeItem *items, int n_items, int partition, It
   return off;
 }
 
-// Host-side enumeration of one item's (sequence, unit) pairs, in the order the
+// Host-side enumeration of one item's (sequence, unit) pairs, in the classes the
 // device-side enumeration (locate_pair_small) uses: remainder units of split
 // contexts, their other units, then the contexts with a single unit.  Appends
 // to out[*n]; false when they do not fit the kernel argument's table or its
@@ -1211,46 +1307,53 @@ bool enumerate_pairs_on_host(const int32_t *ctx_host, int B, int max_ctx, int pa
       for (int j = 0; j < su.nb; ++j)
         if (!push(s, j, c)) return false;
   }
+  // The single-unit contexts end the item (and the last item's end the launch):
+  // longest first, so that what is still running at the very end is short.  The
+  // units are the same in any order, and so are the results.
+  const int first_single = at;
   for (int s = 0; s < B; ++s) {
     const int c = clamped(s);
     if (c > 0 && seq_units(c, partition, rounds, absorb).count() == 1 && !push(s, 0, c)) return false;
   }
+  std::stable_sort(out + first_single, out + at, [](const uint2 &a, const uint2 &b) { return a.y > b.y; });
   *n = at;
   return true;
 }
 
 template <typename T, int BS, int G>
-hipError_t launch_g(const DecodeParams &P, int grid, hipStream_t st) {
+hipError_t launch_g(const DecodeParams &P, int grid, bool sweep, hipStream_t st) {
   constexpr int NW = kWavesPerGroup;
-  hipLaunchKernelGGL((paged_decode_kernel<T, BS, G, NW>), dim3(grid), dim3(64 * NW), 0, st, P);
+  if (sweep) hipLaunchKernelGGL((paged_decode_sweep_kernel<T, BS, G, NW>), dim3(grid), dim3(64 * NW), 0, st, P);
+  else hipLaunchKernelGGL((paged_decode_kernel<T, BS, G, NW>), dim3(grid), dim3(64 * NW), 0, st, P);
   return hipGetLastError();
 }
 
 template <typename T, int BS, int G>
-hipError_t launch_gqa(const DecodeParams &P, int grid, hipStream_t st) {
+hipError_t launch_gqa(const DecodeParams &P, int grid, bool sweep, hipStream_t st) {
   constexpr int NW = kWavesPerGroup;
-  hipLaunchKernelGGL((paged_decode_gqa_kernel<T, BS, G, NW>), dim3(grid), dim3(64 * NW), 0, st, P);
+  if (sweep) hipLaunchKernelGGL((paged_decode_gqa_sweep_kernel<T, BS, G, NW>), dim3(grid), dim3(64 * NW), 0, st, P);
+  else hipLaunchKernelGGL((paged_decode_gqa_kernel<T, BS, G, NW>), dim3(grid), dim3(64 * NW), 0, st, P);
   return hipGetLastError();
 }
 
 template <typename T, int BS>
-hipError_t launch_main(int G, const DecodeParams &P, int grid, hipStream_t st) {
+hipError_t launch_main(int G, const DecodeParams &P, int grid, bool sweep, hipStream_t st) {
   switch (G) {
-    case 1: return launch_g<T, BS, 1>(P, grid, st);
-    case 2: return launch_g<T, BS, 2>(P, grid, st);
-    case 4: return launch_gqa<T, BS, 4>(P, grid, st);
-    case 8: return launch_gqa<T, BS, 8>(P, grid, st);
-    case 16: return launch_gqa<T, BS, 16>(P, grid, st);
+    case 1: return launch_g<T, BS, 1>(P, grid, sweep, st);
+    case 2: return launch_g<T, BS, 2>(P, grid, sweep, st);
+    case 4: return launch_gqa<T, BS, 4>(P, grid, sweep, st);
+    case 8: return launch_gqa<T, BS, 8>(P, grid, sweep, st);
+    case 16: return launch_gqa<T, BS, 16>(P, grid, sweep, st);
     default: return hipErrorInvalidValue;
   }
 }
 
 template <typename T>
-hipError_t launch_bs(int BS, int G, const DecodeParams &P, int grid, hipStream_t st) {
+hipError_t launch_bs(int BS, int G, const DecodeParams &P, int grid, bool sweep, hipStream_t st) {
   switch (BS) {
-    case 8: return launch_main<T, 8>(G, P, grid, st);
-    case 16: return launch_main<T, 16>(G, P, grid, st);
-    case 32: return launch_main<T, 32>(G, P, grid, st);
+    case 8: return launch_main<T, 8>(G, P, grid, sweep, st);
+    case 16: return launch_main<T, 16>(G, P, grid, sweep, st);
+    case 32: return launch_main<T, 32>(G, P, grid, sweep, st);
     default: return hipErrorInvalidValue;
   }
 }
@@ -1396,6 +1499,7 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
       if (host_pairs) P.n_host_pairs = n_pairs;
     }
     int64_t work = 0;
+    bool tightened = false;
     for (int i = first; i < n_items; ++i) {
       if (done[i]) continue;
       const MuxDecodeItem &it = items[i];
@@ -1431,13 +1535,14 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
         continue;
       }
       if (plan[i].table_off != 0) {
-        if (plan[i].units > 0x7fffffff) return MUXA_EUNSUPPORTED;
+        const int64_t rows = static_cast<int64_t>(it.num_seqs) * plan[i].max_splits;
+        if (rows > 0x7fffffff) return MUXA_EUNSUPPORTED;
         PlanItem &t = PP.it[n_tables++];
         t.ctx = it.context_lens;
         t.table = reinterpret_cast<int4 *>(ws + plan[i].table_off);
         t.B = it.num_seqs;
         t.max_ctx = it.max_context_len;
-        t.capacity = static_cast<int32_t>(plan[i].units);
+        t.capacity = static_cast<int32_t>(rows);
         d.unit_table = t.table;
       }
       d.B = it.num_seqs;
@@ -1449,6 +1554,9 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
       d.max_ctx = it.max_context_len;
       d.work_begin = static_cast<int32_t>(work);
       d.scale_log2 = it.scale * 1.4426950408889634f;
+      if (plan[i].units > 0x7fffffff) return MUXA_EUNSUPPORTED;
+      d.pair_begin = static_cast<int32_t>(plan[i].units);       // pairs with a place in the grid
+      if (plan[i].units < static_cast<int64_t>(it.num_seqs) * plan[i].max_splits) tightened = true;
       work += plan[i].units * (it.num_q_heads / G);
       if (work > 0x7fffffff) return MUXA_EUNSUPPORTED;
     }
@@ -1459,9 +1567,22 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
       if (pe != hipSuccess) return hip_fail(pe);
     }
     const int grid = static_cast<int>(work);
-    hipError_t e = dtype == MUXA_DTYPE_F16 ? launch_bs<F16>(block_size, G, P, grid, st)
-                                           : launch_bs<BF16>(block_size, G, P, grid, st);
+    hipError_t e = dtype == MUXA_DTYPE_F16 ? launch_bs<F16>(block_size, G, P, grid, false, st)
+                                           : launch_bs<BF16>(block_size, G, P, grid, false, st);
     if (e != hipSuccess) return hip_fail(e);
+    // Where the caller's bound on the sum of the context lengths made the grid
+    // smaller than the shapes allow, the pairs it may have left out are swept
+    // up behind the launch: one workgroup per item and head group.
+    if (tightened) {
+      int sweep_grid = 0;
+      for (int k = 0; k < P.n_items; ++k) {
+        P.it[k].work_begin = sweep_grid;
+        sweep_grid += P.it[k].Hq / G;
+      }
+      e = dtype == MUXA_DTYPE_F16 ? launch_bs<F16>(block_size, G, P, sweep_grid, true, st)
+                                  : launch_bs<BF16>(block_size, G, P, sweep_grid, true, st);
+      if (e != hipSuccess) return hip_fail(e);
+    }
   }
   return MUXA_OK;
 }

@@ -87,35 +87,48 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout.strip() == ""
 
 
-def test_grid_bound_from_the_context_sum_covers_every_pair():
-    """The host-side sum of context lengths tightens the number of (sequence,
-    partition) pairs a launch reserves.  The reservation is visible, without a
-    GPU, in the workspace size of a batch large enough to need a pair table
-    (16 bytes per reserved pair): for random batches it must never be smaller
-    than the true number of pairs, and never looser than floor(sum / partition)
-    + sequences (the table is rounded up to 256 bytes = 16 pairs)."""
+def test_workspace_size_does_not_depend_on_the_hint_and_host_pairs_are_exact():
+    """The caller's bound on the sum of the context lengths sizes the grid of a
+    device-enumerated launch and nothing else: the pair table of a large batch
+    has a row for every pair the shapes allow, so a bound that is too small can
+    not make the table too small.  The host-side enumeration (the pairs carried
+    in the kernel argument) is exact: for random batches it counts one unit per
+    started partition, less the remainders of at most 16 tokens, which ride on
+    the unit before them."""
     import numpy as np
     lib = _lib.attn()
     rng = np.random.Generator(np.random.PCG64(11))
     for partition in (64, 256, 512):
         for trial in range(20):
-            B = 16 * int(rng.integers(17, 40))      # a multiple of 16: the loose table has no rounding pad
+            B = 16 * int(rng.integers(17, 40))
             hi = int(rng.choice([partition // 2, partition, 3 * partition, 2000]))
-            ctx = rng.integers(0, hi + 1, size=B).astype(np.int64)
+            ctx = rng.integers(0, hi + 1, size=B).astype(np.int32)
             it = _lib.MuxDecodeItem()
             it.num_seqs, it.num_q_heads, it.num_kv_heads = B, 4, 4
             it.num_layers, it.layer = 1, 0
             it.max_context_len = int(ctx.max())
             it.max_blocks = (it.max_context_len + 15) // 16
-            it.total_context_len = 0
-            loose = lib.mux_paged_decode_workspace_bytes(ctypes.addressof(it), 1, partition)
-            it.total_context_len = int(ctx.sum())
-            tight = lib.mux_paged_decode_workspace_bytes(ctypes.addressof(it), 1, partition)
+            sizes = set()
+            for hint in (0, 1, int(ctx.sum()) // 2, int(ctx.sum()), 10 * int(ctx.sum())):
+                it.total_context_len = hint
+                sizes.add(lib.mux_paged_decode_workspace_bytes(ctypes.addressof(it), 1, partition))
+            assert len(sizes) == 1, (partition, trial, sizes)
             max_splits = max(1, -(-it.max_context_len // partition))
-            reserved = B * max_splits - (loose - tight) // 16          # pairs reserved with the hint, rounded up to 16
-            true_pairs = int((-(-ctx // partition)).sum())
-            assert reserved >= true_pairs, (partition, trial, reserved, true_pairs)
-            assert reserved <= min(B * max_splits, int(ctx.sum()) // partition + B) + 15
+            assert sizes.pop() >= (1 << 20) + B * max_splits * 16
+    for partition in (64, 256):
+        for trial in range(20):
+            B = int(rng.integers(1, 40))
+            ctx = rng.integers(0, 4 * partition, size=B).astype(np.int32)
+            it = _lib.MuxDecodeItem()
+            it.num_seqs, it.num_q_heads, it.num_kv_heads, it.num_layers = B, 2, 2, 1
+            it.max_context_len = max(int(ctx.max()), 1)
+            it.max_blocks = (it.max_context_len + 15) // 16
+            it.context_lens_host = ctx.ctypes.data
+            want = 0
+            for c in ctx.tolist():
+                fg, rem = divmod(c, partition)
+                want += fg + (1 if rem > 0 and not (fg > 0 and rem <= 16) else 0)
+            assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, partition) == (want if want <= 384 else 0)
 
 
 # ---------------------------------------------------------------------------

@@ -520,6 +520,44 @@ def test_decode_config2_full_size_pool(full_size_pool_memory):
         _check(m.out[:m.batch].float().cpu(), want)
 
 
+@pytest.mark.parametrize("Hq,Hkv,B,partition", [(2, 2, 9, 64), (8, 1, 7, 128), (1, 1, 300, 64)])
+def test_decode_with_an_understated_sum_of_context_lengths_is_slow_not_wrong(Hq, Hkv, B, partition):
+    """The caller's bound on the sum of the context lengths sizes the grid.  A
+    bound that is far too small leaves most units without a workgroup of their
+    own; the workgroups of the last unit that has one run them.  The outputs must
+    match the oracle, and the NEXT launch on the same workspace - with a correct
+    bound - must too (the arrival counters of the split contexts are back at
+    zero).  Vector-ALU kernel, matrix-core kernel, and a batch large enough for
+    the pair table."""
+    _announce(f"decode, understated context sum Hq={Hq} Hkv={Hkv} B={B}")
+    bs = 16
+    rng = np.random.Generator(np.random.PCG64(77))
+    g = torch.Generator().manual_seed(77)
+    ctx = rng.integers(1, 5 * partition, size=B).astype(np.int32)
+    nblk = (ctx.astype(np.int64) + bs - 1) // bs
+    need = int(nblk.sum()) * Hkv
+    N = need + 5
+    bt, _ = workloads.build_tables(ctx, Hkv, bs, rng.permutation(N)[:need])
+    k_pool, v_pool = orc.allocate_pool(N, bs, torch.float16)
+    k_pool.copy_(torch.randn(k_pool.shape, generator=g).half())
+    v_pool.copy_(torch.randn(v_pool.shape, generator=g).half())
+    pad = (B + 7) // 8 * 8
+    q = torch.randn((pad, Hq * HEAD_SIZE), generator=g).half()
+    scale = HEAD_SIZE ** -0.5
+    want = orc.paged_decode(q, k_pool, v_pool, torch.from_numpy(bt), ctx, scale)
+    dq, dk, dv = q.to(DEV), k_pool.to(DEV), v_pool.to(DEV)
+    dbt, dctx = torch.from_numpy(bt).to(DEV), torch.from_numpy(ctx).to(DEV)
+    out = torch.full((pad, Hq * HEAD_SIZE), 7.0, dtype=torch.float16, device=DEV)
+    ws = torch.zeros((64 << 20,), dtype=torch.uint8, device=DEV)
+    for hint in (1, int(ctx.sum()) // 3, int(ctx.sum())):        # two understated sums, then the true one
+        out.fill_(7.0)
+        ops.paged_decode(out, dq, dk, dv, dbt, dctx, int(ctx.max()), scale, partition_size=partition,
+                         total_context_len=hint, workspace=ws)
+        torch.cuda.synchronize()
+        _check(out[:B].float().cpu(), want)
+        assert int(ws[:1 << 20].view(torch.int32).abs().max().item()) == 0, "arrival counters must be back at zero"
+
+
 @pytest.mark.parametrize("n_pairs", [384, 385])
 def test_decode_at_the_limit_of_host_enumerated_pairs(n_pairs):
     """The kernel argument holds 384 (sequence, unit) pairs.  A batch with
@@ -529,7 +567,7 @@ def test_decode_at_the_limit_of_host_enumerated_pairs(n_pairs):
     from muxserve_amd import _lib
     _announce(f"decode with {n_pairs} pairs")
     # 128 sequences of three units (two full partitions and a remainder) are 384 pairs
-    ctx = [2 * 256 + 1 + (7 * i) % 200 for i in range(128)]
+    ctx = [2 * 256 + 17 + (7 * i) % 200 for i in range(128)]        # remainders of 17 .. 216 tokens: units of their own
     if n_pairs == 385:
         ctx.append(33)
     dev_got, want = _decode_case(41, ctx, 1, 1, 16, partition=256)
