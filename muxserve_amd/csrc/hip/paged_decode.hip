@@ -1432,11 +1432,10 @@ int32_t mux_paged_decode_workspace_init(void *workspace, size_t workspace_bytes,
 namespace mux {
 namespace {
 
-int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
-                          const void *k_pool, const void *v_pool, int64_t num_pool_blocks,
-                          int32_t head_size, int32_t block_size, int32_t dtype,
-                          int32_t partition_size, void *workspace, size_t workspace_bytes,
-                          void *stream) {
+// Everything about a call that can be refused before anything is launched.
+int32_t validate_call(const MuxDecodeItem *items, int32_t n_items, const void *k_pool, const void *v_pool,
+                      int64_t num_pool_blocks, int32_t head_size, int32_t block_size, int32_t dtype,
+                      int32_t partition_size) {
   if (!items || n_items <= 0 || n_items > MUXA_MAX_DECODE_ITEMS) return MUXA_EINVAL;
   if (!k_pool || !v_pool || num_pool_blocks <= 0) return MUXA_EINVAL;
   if ((reinterpret_cast<uintptr_t>(k_pool) & 15u) || (reinterpret_cast<uintptr_t>(v_pool) & 15u))
@@ -1449,6 +1448,17 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
     const int32_t rc = validate_item(items[i], block_size);
     if (rc != MUXA_OK) return rc;
   }
+  return MUXA_OK;
+}
+
+int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
+                          const void *k_pool, const void *v_pool, int64_t num_pool_blocks,
+                          int32_t head_size, int32_t block_size, int32_t dtype,
+                          int32_t partition_size, void *workspace, size_t workspace_bytes,
+                          void *stream) {
+  const int32_t vrc = validate_call(items, n_items, k_pool, v_pool, num_pool_blocks, head_size, block_size, dtype,
+                                    partition_size);
+  if (vrc != MUXA_OK) return vrc;
   const int partition = choose_partition(items, n_items, partition_size);
   const DecodePolicy pol = choose_policy(items, n_items, partition);
   const int rounds = pol.rounds, absorb = pol.absorb;
@@ -1641,12 +1651,10 @@ int32_t mux_multi_decode_noalloc(const MuxDecodeItem *items, int32_t n_items,
                                  int32_t head_size, int32_t block_size, int32_t dtype,
                                  int32_t partition_size, void *stream) {
   using namespace mux;
-  if (!items || n_items <= 0 || n_items > MUXA_MAX_DECODE_ITEMS) return MUXA_EINVAL;
-  if (partition_size < 0 || partition_size % 64 != 0) return MUXA_EINVAL;
-  for (int i = 0; i < n_items; ++i)
-    if (items[i].num_kv_heads <= 0 || items[i].num_q_heads <= 0 || items[i].num_seqs < 0 ||
-        items[i].max_context_len < 0 || items[i].total_context_len < 0)
-      return MUXA_EINVAL;
+  // Every check the launch makes is made first: a refused call has launched nothing.
+  const int32_t vrc = validate_call(items, n_items, k_pool, v_pool, num_pool_blocks, head_size, block_size, dtype,
+                                    partition_size);
+  if (vrc != MUXA_OK) return vrc;
   // The call's scratch need against the fixed size of the static array.
   const int partition = choose_partition(items, n_items, partition_size);
   const size_t need = plan_workspace(items, n_items, partition, nullptr);

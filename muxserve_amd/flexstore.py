@@ -19,10 +19,19 @@ Answered exactly as the reference frames them:
   the start-up bookkeeping: "get_rank", "init_finished",
   "query_num_ready_processes", "start_warmup", "warmup_ready"  manager.py:762-783
   "log_stats" -> None, "exit" -> None and the handler is closed  manager.py:820-827
-Requests whose answer is a GPU memory handle to open in another process -
-"weight", "cache_init", "lock_init" (manager.py:784-806) - raise
-IpcExportExcluded: exporting the pool across processes is not part of this
-build.  A request type outside the reference's list is answered with the
+  ("cache_init", [rank, model_name])                   manager.py:789-793
+      -> (metadata of the K pool, metadata of the V pool) as get_tensor_metadata
+         makes it (manager.py:893-911): the IPC handle of the pool's storage
+         plus sizes, strides, dtype - what the runtime side hands to
+         torch.multiprocessing.reductions.rebuild_cuda_tensor, as the reference's
+         model_loader.py:46 does with the weights.  Answered only when the handler
+         was given the pool tensors and each stays under MAX_IPC_BYTES: a shared
+         allocation of 2 GiB or more cannot be opened by another process on the
+         hosts this build runs on, so a pool of that size raises
+         IpcExportExcluded instead.
+Requests for the other GPU memory handles - "weight", "lock_init"
+(manager.py:784-806) - raise IpcExportExcluded: model weights and the lock
+tensor are not part of this build.  A request type outside the reference's list is answered with the
 string "Incorrect format" (manager.py:756-759); one that is in the list but has
 no branch in the loop ("blocktable_load", "blocktable_store") raises
 RuntimeError("Unknown request type") as the reference does (manager.py:828-830).
@@ -40,7 +49,44 @@ INCORRECT_FORMAT = "Incorrect format"
 
 
 class IpcExportExcluded(NotImplementedError):
-    """The request asks for a GPU memory handle for another process."""
+    """The request asks for a GPU memory handle this build does not export."""
+
+
+# Shared device allocations of 2 GiB and more do not open in a second process here.
+MAX_IPC_BYTES = (2 << 30) - 1
+
+
+def tensor_metadata(tensor) -> Dict[str, Any]:
+    """What another process needs to map `tensor`'s memory: the fields of
+    get_tensor_metadata (muxserve/flexstore/manager.py:893-911), which are the
+    keyword arguments of torch.multiprocessing.reductions.rebuild_cuda_tensor.
+    The tensor's storage must stay alive in this process while others use it."""
+    storage = tensor.untyped_storage()
+    t = storage._share_cuda_()
+    return {
+        "tensor_size": tensor.size(),
+        "tensor_stride": tensor.stride(),
+        "tensor_offset": tensor.storage_offset(),
+        "storage_cls": type(storage),
+        "dtype": tensor.dtype,
+        "storage_device": t[0],
+        "storage_handle": t[1],
+        "storage_size_bytes": t[2],
+        "storage_offset_bytes": t[3],
+        "requires_grad": tensor.requires_grad,
+        "ref_counter_handle": t[4],
+        "ref_counter_offset": t[5],
+        "event_handle": t[6],
+        "event_sync_required": t[7],
+    }
+
+
+def rebuild_tensor(metadata: Dict[str, Any]):
+    """The runtime side of tensor_metadata: a tensor over the other process's
+    memory (muxserve/flexserver/model_loader.py:46)."""
+    import torch
+    from torch.multiprocessing.reductions import rebuild_cuda_tensor
+    return rebuild_cuda_tensor(torch.Tensor, **metadata)
 
 
 class CacheRequestHandler:
@@ -48,7 +94,11 @@ class CacheRequestHandler:
     heads) and occupancy, the start-up counters."""
 
     def __init__(self, storage, model_cache_info: Dict[str, Tuple[int, int]], num_gpu_blocks: int,
-                 num_runtime_processes: int = 1, rank: int = 0, local_world_size: int = 1):
+                 num_runtime_processes: int = 1, rank: int = 0, local_world_size: int = 1, gpu_cache=None):
+        """gpu_cache: optional (k_pool, v_pool) device tensors this process owns;
+        with them "cache_init" is answered (pools under MAX_IPC_BYTES each)."""
+        self.gpu_cache = gpu_cache
+        self._gpu_cache_metadata = None
         self.block_manager = storage
         self.model_cache_info = {k: (int(v[0]), int(v[1])) for k, v in model_cache_info.items()}
         self.model_occupy_info = {k: 0 for k in self.model_cache_info}
@@ -106,8 +156,19 @@ class CacheRequestHandler:
         if kind == "exit":
             self.closed = True
             return None
-        if kind in ("weight", "cache_init", "lock_init"):
-            raise IpcExportExcluded(f"{kind}: GPU memory handles for other processes are not exported by this build")
+        if kind == "cache_init":
+            if self.gpu_cache is None:
+                raise IpcExportExcluded("cache_init: this handler was not given the pool tensors")
+            if self._gpu_cache_metadata is None:          # once, as at manager.py:390-393
+                for t in self.gpu_cache:
+                    if t.untyped_storage().nbytes() > MAX_IPC_BYTES:
+                        raise IpcExportExcluded(
+                            f"cache_init: a pool tensor of {t.untyped_storage().nbytes()} bytes cannot be opened by "
+                            f"another process here (shared allocations stay under {MAX_IPC_BYTES + 1} bytes)")
+                self._gpu_cache_metadata = tuple(tensor_metadata(t) for t in self.gpu_cache)
+            return self._gpu_cache_metadata
+        if kind in ("weight", "lock_init"):
+            raise IpcExportExcluded(f"{kind}: not exported by this build (no model weights, no lock tensor)")
         raise RuntimeError("Unknown request type")
 
     def cache_alloc_for(self, model_name: str):

@@ -38,10 +38,18 @@ def _run_both(models, dk, dv, partition):
     ref = [m.out.clone() for m in models]
     for m in models:
         m.out.fill_(7.0)
-    before = torch.cuda.memory_allocated()
+    # (a first call outside the check: the first launch of a kernel loads its code object)
     ops.multi_decode_noalloc(calls, dk, dv, partition_size=partition)
     torch.cuda.synchronize()
+    for m in models:
+        m.out.fill_(7.0)
+    torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+    ops.multi_decode_noalloc(calls, dk, dv, partition_size=partition)
+    torch.cuda.synchronize()
+    # neither torch's allocator nor the device's free memory (which a hipMalloc inside the library would move)
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     return ref, [m.out.clone() for m in models]
 
 
@@ -97,3 +105,28 @@ def test_noalloc_decode_refuses_what_the_static_array_cannot_hold():
         ops.multi_decode_noalloc([call], dk, dv, partition_size=256)
     torch.cuda.synchronize()
     assert (out == 7.0).all(), "a refused call must not launch anything"
+
+
+def test_noalloc_decode_refused_for_its_arguments_launches_nothing():
+    """A call that is refused for a malformed argument (here: a block size the
+    library does not have, then a table too narrow for max_context_len) must
+    not have launched anything - not even the fill kernel that clears the
+    static array's arrival counters."""
+    print("[case] no-alloc decode: refused arguments", flush=True)
+    import ctypes
+    lib = _lib.attn()
+    bs = 16
+    dk, dv = allocate_gpu_cache(64, bs, DEV)
+    q = torch.zeros((8, 4 * 128), dtype=torch.float16, device=DEV)
+    out = torch.full_like(q, 7.0)
+    bt = torch.zeros((1, 8, 4, 40), dtype=torch.int32, device=DEV)
+    cl = torch.full((8,), 600, dtype=torch.int32, device=DEV)
+    items = (_lib.MuxDecodeItem * 1)(ops.DecodeCall(out, q, bt, cl, 600, 1.0).to_item())
+    st = torch.cuda.current_stream().cuda_stream
+    rc = lib.mux_multi_decode_noalloc(ctypes.addressof(items), 1, dk.data_ptr(), dv.data_ptr(), 64, 128, 24, 0, 128, st)
+    assert rc == -2
+    items[0].max_blocks = 10                      # 160 tokens of table for 600-token contexts
+    rc = lib.mux_multi_decode_noalloc(ctypes.addressof(items), 1, dk.data_ptr(), dv.data_ptr(), 64, 128, bs, 0, 128, st)
+    assert rc == -1
+    torch.cuda.synchronize()
+    assert (out == 7.0).all()
