@@ -285,9 +285,21 @@ def bench_cache_write(args):
     ms_p = _time(write, args.steps, args.warmup)
     ms_warm = _time(lambda _: write(0), args.steps, args.warmup)
     bytes_p = workloads.cache_write_bytes(T, 52)
+    # The yardstick: a contiguous copy of as many bytes in and out (the probe library's copy
+    # kernel, and the framework's), rotated over buffers the same way.
+    from muxserve_amd import _lib as _l
+    half = T * 52 * 2 * D * 2
+    srcs = [kv for kv, _ in psets]
+    dsts = [torch.empty((half,), dtype=torch.uint8, device=dev) for _ in psets]
+    st = torch.cuda.current_stream().cuda_stream
+    ms_copy = _time(lambda i: _l.probe().mux_probe_copy(dsts[i % 5].data_ptr(), srcs[i % 5].data_ptr(), half, st),
+                    args.steps, args.warmup)
+    ms_tcopy = _time(lambda i: dsts[i % 5].copy_(srcs[i % 5].view(torch.uint8).view(-1)), args.steps, args.warmup)
     gbs = bytes_p / (ms_p * 1e-3) / 1e9
     cfg = {"workload": "cache_write", "prefill_shape": "52 heads x 4096 tokens", "prefill_bytes": bytes_p,
            "same_buffers_every_step_ms": ms_warm, "same_buffers_every_step_gbs": bytes_p / (ms_warm * 1e-3) / 1e9,
+           "contiguous_copy_of_the_same_bytes": {"probe_copy_ms": ms_copy, "probe_copy_gbs": 2 * half / (ms_copy * 1e-3) / 1e9,
+                                                 "torch_copy_ms": ms_tcopy, "torch_copy_gbs": 2 * half / (ms_tcopy * 1e-3) / 1e9},
            "decode_shape": "7b/13b/30b, 56 tokens, three launches", "decode_ms": ms_d, "decode_bytes": bytes_d,
            "decode_gbs": bytes_d / (ms_d * 1e-3) / 1e9,
            "decode_one_fused_launch_ms": ms_d1, "decode_one_fused_launch_with_rope_ms": ms_dr,

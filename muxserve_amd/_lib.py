@@ -198,6 +198,8 @@ def probe():
         lib = _open(PROBE_LIB_PATH)
         lib.mux_probe_gather_read.restype = c_i32
         lib.mux_probe_gather_read.argtypes = [c_vp, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp]
+        lib.mux_probe_copy.restype = c_i32
+        lib.mux_probe_copy.argtypes = [c_vp, c_vp, c_i64, c_vp]
         lib.mux_probe_where.restype = c_i32
         lib.mux_probe_where.argtypes = [c_vp, c_i32, c_i32, c_vp]
         _probe = lib

@@ -110,6 +110,8 @@ __device__ __forceinline__ void cache_write_window(
   const int i = threadIdx.x & 15;
   const int c = threadIdx.x >> 4;
   const int64_t pool_slots = num_blocks * block_size;
+  // Block sizes are powers of two (8, 16, 32): slot -> (block, offset) by shift and mask.
+  const int bs_shift = __builtin_ctz(static_cast<unsigned>(block_size));
 
   // Slots of tokens T0-16 .. T0+31 (bit j of the masks below is token T0-16+j);
   // -1 for tokens outside the batch, skipped tokens and slots outside the pool
@@ -240,8 +242,8 @@ __device__ __forceinline__ void cache_write_window(
     const int j = ja + 16 * pass + i;
     const int64_t slot = j < jb ? s_slot[j] : -1;
     if (slot >= 0) {
-      const int64_t blk = slot / block_size;
-      const int o = static_cast<int>(slot - blk * block_size);
+      const int64_t blk = slot >> bs_shift;
+      const int o = static_cast<int>(slot) & (block_size - 1);
       // Element path for tokens that no run covers (a run starts at most 7 tokens back).
       const unsigned long long cover = in_win & (0xffull << (j > 7 ? j - 7 : 0)) & ~(~0ull << (j + 1));
       store16(&k_pool[(blk * (D / 8) + c) * block_size + o], *reinterpret_cast<const uint4 *>(&kt[j][c * 8]),
@@ -269,8 +271,8 @@ __device__ __forceinline__ void cache_write_window(
     for (int e = 0; e < 4; ++e)
       w[e] = static_cast<uint32_t>(vt[jp + 2 * e][d]) | (static_cast<uint32_t>(vt[jp + 2 * e + 1][d]) << 16);
     const int64_t slot0 = s_slot[jp];
-    const int64_t b0 = slot0 / block_size;
-    const int o0 = static_cast<int>(slot0 - b0 * block_size);
+    const int64_t b0 = slot0 >> bs_shift;
+    const int o0 = static_cast<int>(slot0) & (block_size - 1);
     store16(v_pool + (b0 * D + d) * block_size + o0, make_uint4(w[0], w[1], w[2], w[3]), rows_complete);
   }
 }

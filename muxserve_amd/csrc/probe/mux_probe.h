@@ -31,6 +31,11 @@ int32_t mux_probe_gather_read(const void *k_pool, const void *v_pool, int64_t nu
  * spreads over every compute unit its stream may use. */
 int32_t mux_probe_where(uint32_t *out, int32_t num_workgroups, int32_t spin_microseconds, void *stream);
 
+/* Copies nbytes (a multiple of 16; both pointers 16-byte aligned) from src to
+ * dst with non-temporal 16-byte loads and stores, one chunk per thread: the
+ * yardstick for kernels that read and write equal amounts (the cache write). */
+int32_t mux_probe_copy(void *dst, const void *src, int64_t nbytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
