@@ -272,16 +272,28 @@ __device__ __forceinline__ void consume_tile(uint4 (&kreg)[16], uint4 (&vreg)[Ge
     s[g] = valid ? (a0 + a1) * scale_log2 : -INFINITY;
   }
 
+  // fp16: the probabilities go to the P.V product as packed halves, one
+  // v_dot2_f32_f16 per pair of tokens instead of two conversions and two
+  // multiply-adds (a quarter of the product's instructions; the accumulation stays
+  // fp32).  They are taken 2^15 times too large, so that the smallest half-precision
+  // normal stands for a probability of 2e-9 rather than 6e-5; the running sum
+  // carries the same factor, which therefore cancels in every ratio this kernel and
+  // the merges form.  bf16 would keep 8 bits of a probability: it stays on the
+  // fp32 path.
+  constexpr bool kHalfP = __is_same(T, F16);
+  constexpr float kPShift = kHalfP ? 15.f : 0.f;
+  uint16_t(*p_h)[64] = reinterpret_cast<uint16_t(*)[64]>(p_w);     // the same LDS, as halves, one row per head
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     const float m_new = fmaxf(m[g], wave_max(s[g]));
     const float alpha = fast_exp2(m[g] - m_new);
-    const float p = fast_exp2(s[g] - m_new);
+    const float p = fast_exp2(s[g] - m_new + kPShift);
     l[g] = l[g] * alpha + p;
 #pragma unroll
     for (int j = 0; j < Geo::VI; ++j) acc[g][j] *= alpha;
     m[g] = m_new;
-    p_w[g][lane] = p;
+    if constexpr (kHalfP) p_h[2 * g][lane] = f32_to_f16_bits(p);     // (row 2 g: rows are 128 bytes, a float row 256)
+    else p_w[g][lane] = p;
   }
   wave_lds_sync();
 
@@ -289,16 +301,29 @@ __device__ __forceinline__ void consume_tile(uint4 (&kreg)[16], uint4 (&vreg)[Ge
   for (int b = 0; b < Geo::BPT; ++b) {
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      const float4 pa = *reinterpret_cast<const float4 *>(&p_w[g][b * BS + part * 8]);
-      const float4 pb = *reinterpret_cast<const float4 *>(&p_w[g][b * BS + part * 8 + 4]);
+      if constexpr (kHalfP) {
+        const uint4 pp = *reinterpret_cast<const uint4 *>(&p_h[2 * g][b * BS + part * 8]);
 #pragma unroll
-      for (int j = 0; j < Geo::VI; ++j) {
-        float a = acc[g][j];
-        a = fma2<T>(vreg[b][j].x, pa.x, pa.y, a);
-        a = fma2<T>(vreg[b][j].y, pa.z, pa.w, a);
-        a = fma2<T>(vreg[b][j].z, pb.x, pb.y, a);
-        a = fma2<T>(vreg[b][j].w, pb.z, pb.w, a);
-        acc[g][j] = a;
+        for (int j = 0; j < Geo::VI; ++j) {
+          float a = acc[g][j];
+          a = dot2<T>(vreg[b][j].x, pp.x, a);
+          a = dot2<T>(vreg[b][j].y, pp.y, a);
+          a = dot2<T>(vreg[b][j].z, pp.z, a);
+          a = dot2<T>(vreg[b][j].w, pp.w, a);
+          acc[g][j] = a;
+        }
+      } else {
+        const float4 pa = *reinterpret_cast<const float4 *>(&p_w[g][b * BS + part * 8]);
+        const float4 pb = *reinterpret_cast<const float4 *>(&p_w[g][b * BS + part * 8 + 4]);
+#pragma unroll
+        for (int j = 0; j < Geo::VI; ++j) {
+          float a = acc[g][j];
+          a = fma2<T>(vreg[b][j].x, pa.x, pa.y, a);
+          a = fma2<T>(vreg[b][j].y, pa.z, pa.w, a);
+          a = fma2<T>(vreg[b][j].z, pb.x, pb.y, a);
+          a = fma2<T>(vreg[b][j].w, pb.z, pb.w, a);
+          acc[g][j] = a;
+        }
       }
     }
   }
