@@ -30,14 +30,15 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0     # dense fp16 / bf16
 # HBM bytes moved per algorithmic byte by the decode kernel on this workload,
 # from the FETCH_SIZE / WRITE_SIZE counter passes summarised in
-# profiles/paged_decode_mixed3_hbm_traffic.txt (421.0 MB measured / 410.6 MB).
-MIXED3_TRAFFIC_RATIO = 1.025
+# profiles/paged_decode_mixed3_hbm_traffic.txt (420.6 MB measured / 410.6 MB).
+MIXED3_TRAFFIC_RATIO = 1.024
 # Same for the grouped-query decode kernel (profiles/paged_decode_gqa_long_kernel_trace_and_traffic.txt:
-# 1394.5 MB / 1358.8 MB) and the prefill-shaped cache write (profiles/other_kernels_kernel_trace.txt:
-# 231.9 MB / 219.8 MB).
-GQA_LONG_TRAFFIC_RATIO = 1.026
+# 1390.0 MB / 1358.8 MB) and the prefill-shaped cache write
+# (profiles/reshape_and_cache_write_kernel_trace_and_traffic.txt: 231.9 MB / 219.8 MB).
+GQA_LONG_TRAFFIC_RATIO = 1.023
 CACHE_WRITE_TRAFFIC_RATIO = 1.055
 
 
@@ -61,7 +62,7 @@ def parse():
     ap.add_argument("--unfused", action="store_true", help="one launch per model instead of one fused launch")
     ap.add_argument("--workload", default="mixed3_decode",
                     choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long", "model_ops", "host_step",
-                             "cu_masks", "prefill_long", "decode_timeline"],
+                             "cu_masks", "prefill_long", "decode_timeline", "mfma_ceiling"],
                     help="mixed3_decode is the headline metric; the others are the remaining synthetic "
                          "shapes, each printing its own JSON line")
     return ap.parse_args()
@@ -306,7 +307,7 @@ def bench_cache_write(args):
            "decode_step_rope_write_attention_two_launches_ms": ms_step}
     roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
             "traffic": bytes_p * CACHE_WRITE_TRAFFIC_RATIO,
-            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiles/other_kernels_kernel_trace.txt",
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiles/reshape_and_cache_write_kernel_trace_and_traffic.txt",
             "kernel": "reshape_and_cache_kernel"}
     return _line("KV-cache write tokens/s (prefill-shaped, 52 heads)", T / (ms_p * 1e-3), "tokens/s", args, ms_p,
                  cfg, roof, dtype="u16")
@@ -402,7 +403,10 @@ def bench_cu_masks(args):
         return set(where)
 
     sets = {}
-    for name, kw in (("percent 0-40", dict(lo_percent=0, hi_percent=40)), ("percent 40-100", dict(lo_percent=40, hi_percent=100)),
+    # The two narrow ranges (mask bits 0-9 and 10-32) show how the driver deals consecutive
+    # mask bits: over the dies first, the shader engines next.
+    for name, kw in (("percent 0-4", dict(lo_percent=0, hi_percent=4)), ("percent 4-13", dict(lo_percent=4, hi_percent=13)),
+                     ("percent 0-40", dict(lo_percent=0, hi_percent=40)), ("percent 40-100", dict(lo_percent=40, hi_percent=100)),
                      ("parts {0}", dict(parts=[0])), ("parts {9}", dict(parts=[9])), ("parts {0,3,7}", dict(parts=[0, 3, 7])),
                      ("parts {1,2,9}", dict(parts=[1, 2, 9])), ("parts {4,5,6,8}", dict(parts=[4, 5, 6, 8]))):
         st = ops.CUMaskedStream(**kw)
@@ -416,6 +420,49 @@ def bench_cu_masks(args):
     return _line("compute units reached through CU-masked streams", float(ncu), "compute units", args, 0.0, cfg,
                  {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": None, "traffic": None,
                   "kernel": "probe_where_kernel (records XCC_ID / HW_ID per workgroup)"}, dtype="u32")
+
+
+def bench_mfma_ceiling(args):
+    """What the matrix cores sustain on this box (v_mfma_f32_32x32x16_f16 from
+    register operands, nothing else in the loop) for one, two and four
+    independent accumulation chains per wave, with vector-ALU work in the same
+    wave and in other waves of the SIMD, and the shader clock each case ran at:
+    the ceiling the causal prefill kernel is read against (probe_mfma_kernel in
+    libmuxprobe.so)."""
+    import torch
+    from muxserve_amd import _lib, ops
+    lib = _lib.probe()
+    ncu, _ = ops.device_cu_info()
+    iters = 40000
+    sink = torch.zeros(1, dtype=torch.float32, device="cuda:0")
+    rows = []
+    # (label, chains, valu per iteration, waves per workgroup, mfma waves, workgroups per CU)
+    cases = [("1 chain, 1 wave per SIMD", 1, 0, 4, 4, 1), ("2 chains, 1 wave per SIMD", 2, 0, 4, 4, 1),
+             ("4 chains, 1 wave per SIMD", 4, 0, 4, 4, 1), ("1 chain, 2 waves per SIMD", 1, 0, 8, 8, 1),
+             ("2 chains, 2 waves per SIMD", 2, 0, 8, 8, 1), ("4 chains, 2 waves per SIMD", 4, 0, 8, 8, 1),
+             ("4 chains + 8 v_fma_f32 per iteration in the same wave", 4, 8, 4, 4, 1),
+             ("4 chains + 32 v_fma_f32 per iteration in the same wave", 4, 32, 4, 4, 1),
+             ("4 chains in one wave, 32 v_fma_f32 per iteration in the SIMD's other wave", 4, 0, 8, 4, 1),
+             ("no MFMA: 32 v_fma_f32 per iteration, 1 wave per SIMD", 4, 0, 4, 0, 1)]
+    for label, chains, valu, waves, mfma_waves, per_cu in cases:
+        n_wg = ncu * per_cu
+        ticks = torch.zeros(n_wg, 2, dtype=torch.int32, device="cuda:0")
+
+        def launch(_i):
+            rc = lib.mux_probe_mfma(chains, valu, iters, n_wg, waves, mfma_waves, ticks.data_ptr(), sink.data_ptr(),
+                                    torch.cuda.current_stream().cuda_stream)
+            if rc != 0:
+                raise RuntimeError(f"mux_probe_mfma returned {rc}")
+        ms = _time(launch, 10, 3)
+        t = ticks.cpu().numpy().astype(np.int64) & 0xffffffff
+        clock_ghz = float(np.median(t[:, 0] / np.maximum(t[:, 1], 1)) * 0.1)
+        flops = float(n_wg) * mfma_waves * iters * chains * 32768.0
+        rows.append({"case": label, "ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "shader_clock_ghz": clock_ghz})
+    best = max(r["tflops"] for r in rows)
+    cfg = {"workload": "mfma_ceiling", "instruction": "v_mfma_f32_32x32x16_f16", "iterations": iters, "cases": rows}
+    roof = {"bound": "mfma", "achieved": best, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": best / MFMA_PEAK_TFLOPS,
+            "traffic": None, "kernel": "probe_mfma_kernel (register operands only)"}
+    return _line("matrix-core rate sustained by independent MFMA chains", best, "TFLOP/s", args, rows[2]["ms"], cfg, roof)
 
 
 def bench_decode_timeline(args):
@@ -769,7 +816,8 @@ def main():
               file=sys.stderr)
         sys.exit(2)
     other = {"prefill3": bench_prefill3, "cache_write": bench_cache_write, "colocated": bench_colocated, "cu_masks": bench_cu_masks, "prefill_long": bench_prefill_long, "decode_timeline": bench_decode_timeline,
-             "gqa_long": bench_gqa_long, "model_ops": bench_model_ops, "host_step": bench_host_step}
+             "gqa_long": bench_gqa_long, "model_ops": bench_model_ops, "host_step": bench_host_step,
+             "mfma_ceiling": bench_mfma_ceiling}
     if args.workload in other:
         print(json.dumps(other[args.workload](args)))
         return

@@ -36,6 +36,18 @@ int32_t mux_probe_where(uint32_t *out, int32_t num_workgroups, int32_t spin_micr
  * yardstick for kernels that read and write equal amounts (the cache write). */
 int32_t mux_probe_copy(void *dst, const void *src, int64_t nbytes, void *stream);
 
+/* What the matrix cores sustain: num_workgroups workgroups of
+ * waves_per_workgroup (1..8) waves; waves below mfma_waves run `iterations`
+ * iterations of `chains` (1, 2 or 4) independent v_mfma_f32_32x32x16_f16
+ * accumulations from register operands (32768 flop each per wave) plus
+ * valu_per_iteration (0; with 4 chains also 8 or 32) dependent v_fma_f32; the
+ * remaining waves run 32 independent v_fma_f32 per iteration and no MFMA.  ticks
+ * (DEVICE uint32 [num_workgroups, 2]) receives per workgroup the shader-clock
+ * ticks and the 100 MHz ticks wave 0's loop took.  sink: DEVICE float [1].
+ * Returns 0, -1 (invalid argument), -2 (combination not built) or -4. */
+int32_t mux_probe_mfma(int32_t chains, int32_t valu_per_iteration, int32_t iterations, int32_t num_workgroups,
+                       int32_t waves_per_workgroup, int32_t mfma_waves, uint32_t *ticks, float *sink, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

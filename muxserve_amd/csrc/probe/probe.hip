@@ -127,3 +127,105 @@ extern "C" int32_t mux_probe_copy(void *dst, const void *src, int64_t nbytes, vo
                      static_cast<const mux::probe_u32x4 *>(src), n);
   return hipGetLastError() == hipSuccess ? 0 : -4;
 }
+
+// ---------------------------------------------------------------------------
+// What the matrix cores sustain, and what they sustain beside vector-ALU work:
+// waves 0 .. mfma_waves-1 of a workgroup run `iters` iterations of CHAINS
+// independent v_mfma_f32_32x32x16_f16 accumulations (operands in registers,
+// nothing else in the loop) plus VALU dependent v_fma_f32 of their own; the
+// other waves run 32 independent v_fma_f32 per iteration and no MFMA.  The
+// figures the causal prefill kernel is priced against: the dense peak is quoted
+// at 2.4 GHz, and under sustained matrix work the shader clock settles lower.
+// Wave 0 of every workgroup reports the shader-clock and 100 MHz-clock ticks its
+// loop took, which gives the clock the chip really ran at.
+// ---------------------------------------------------------------------------
+namespace mux {
+
+typedef _Float16 probe_v8f16 __attribute__((ext_vector_type(8)));
+typedef float probe_v16f32 __attribute__((ext_vector_type(16)));
+
+template <int CHAINS, int VALU>
+__global__ __launch_bounds__(512) void probe_mfma_kernel(int iters, int mfma_waves, uint32_t *__restrict__ ticks,
+                                                         float *sink) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const long long c0 = __builtin_readcyclecounter();
+  const long long r0 = static_cast<long long>(__builtin_amdgcn_s_memrealtime());
+  float folded = 0.f;
+  if (wave < mfma_waves) {
+    probe_v8f16 a, b;
+    // Operands with all mantissa bits in play (a multiplier fed with zeros or small
+    // integers draws less power and would flatter the clock): hashed values in (-1, 1).
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      uint32_t h = (threadIdx.x * 8u + i + blockIdx.x * 4099u) * 2654435761u;
+      h ^= h >> 15;
+      h *= 2246822519u;
+      h ^= h >> 13;
+      a[i] = static_cast<_Float16>(static_cast<float>(static_cast<int>(h & 0xffffu) - 32768) * (1.f / 32768.f));
+      b[i] = static_cast<_Float16>(static_cast<float>(static_cast<int>(h >> 16) - 32768) * (1.f / 32768.f));
+    }
+    probe_v16f32 acc[CHAINS];
+#pragma unroll
+    for (int c = 0; c < CHAINS; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[c][i] = 0.f;
+    float f = static_cast<float>(threadIdx.x), g = 1.0001f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int c = 0; c < CHAINS; ++c) acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[c], 0, 0, 0);
+#pragma unroll
+      for (int v = 0; v < VALU; ++v) f = __builtin_fmaf(f, g, 0.5f);
+      asm volatile("" : "+v"(f));
+    }
+#pragma unroll
+    for (int c = 0; c < CHAINS; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) folded += acc[c][i];
+    folded += f;
+  } else {
+    float f[32];
+#pragma unroll
+    for (int v = 0; v < 32; ++v) f[v] = static_cast<float>(threadIdx.x + v);
+    const float g = 1.0001f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int v = 0; v < 32; ++v) {
+        f[v] = __builtin_fmaf(f[v], g, 0.5f);
+        asm volatile("" : "+v"(f[v]));
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < 32; ++v) folded += f[v];
+  }
+  const long long c1 = __builtin_readcyclecounter();
+  const long long r1 = static_cast<long long>(__builtin_amdgcn_s_memrealtime());
+  if (threadIdx.x == 0) {
+    ticks[2 * blockIdx.x] = static_cast<uint32_t>(c1 - c0);
+    ticks[2 * blockIdx.x + 1] = static_cast<uint32_t>(r1 - r0);
+  }
+  if (folded == 123.456f) sink[0] = folded;     // keeps the loops alive; practically never taken
+}
+
+}  // namespace mux
+
+extern "C" int32_t mux_probe_mfma(int32_t chains, int32_t valu_per_iteration, int32_t iterations,
+                                  int32_t num_workgroups, int32_t waves_per_workgroup, int32_t mfma_waves,
+                                  uint32_t *ticks, float *sink, void *stream) {
+  using namespace mux;
+  if (!ticks || !sink || iterations <= 0 || iterations > (1 << 24) || num_workgroups <= 0) return -1;
+  if (waves_per_workgroup < 1 || waves_per_workgroup > 8 || mfma_waves < 0 || mfma_waves > waves_per_workgroup) return -1;
+  const dim3 grid(static_cast<uint32_t>(num_workgroups)), block(static_cast<uint32_t>(64 * waves_per_workgroup));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define MUX_PROBE_MFMA(C, V)                                                                                  \
+  if (chains == C && valu_per_iteration == V) {                                                                \
+    hipLaunchKernelGGL((probe_mfma_kernel<C, V>), grid, block, 0, st, iterations, mfma_waves, ticks, sink);    \
+    return hipGetLastError() == hipSuccess ? 0 : -4;                                                           \
+  }
+  MUX_PROBE_MFMA(1, 0)
+  MUX_PROBE_MFMA(2, 0)
+  MUX_PROBE_MFMA(4, 0)
+  MUX_PROBE_MFMA(4, 8)
+  MUX_PROBE_MFMA(4, 32)
+#undef MUX_PROBE_MFMA
+  return -2;
+}
