@@ -296,11 +296,30 @@ def bench_cache_write(args):
     ms_copy = _time(lambda i: _l.probe().mux_probe_copy(dsts[i % 5].data_ptr(), srcs[i % 5].data_ptr(), half, st),
                     args.steps, args.warmup)
     ms_tcopy = _time(lambda i: dsts[i % 5].copy_(srcs[i % 5].view(torch.uint8).view(-1)), args.steps, args.warmup)
+    # ... and the same copy with the cache write's own destinations: sources read contiguously,
+    # every 4 KiB written to the pool block the step's slots name (one K and one V block per
+    # workgroup), no windows, no transposition.
+    flat = [kv.view(-1) for kv, _ in psets]
+    blk_ids = [(ds[::bs, 0, :] // bs).reshape(-1).to(torch.int32).contiguous() for _, ds in psets]
+    n_blk = int(blk_ids[0].numel())
+
+    def scatter(i):
+        f, ids = flat[i % 5], blk_ids[i % 5]
+        rc = _l.probe().mux_probe_scatter_copy(k_pool.data_ptr(), v_pool.data_ptr(), N, f.data_ptr(),
+                                               f[n_blk * 2048:].data_ptr(), ids.data_ptr(), n_blk, st)
+        if rc != 0:
+            raise RuntimeError(f"mux_probe_scatter_copy returned {rc}")
+
+    ms_scopy = _time(scatter, args.steps, args.warmup)
+    for i in range(5):          # the pool holds the probe's bytes now: put the step's own back
+        write(i)
     gbs = bytes_p / (ms_p * 1e-3) / 1e9
     cfg = {"workload": "cache_write", "prefill_shape": "52 heads x 4096 tokens", "prefill_bytes": bytes_p,
            "same_buffers_every_step_ms": ms_warm, "same_buffers_every_step_gbs": bytes_p / (ms_warm * 1e-3) / 1e9,
            "contiguous_copy_of_the_same_bytes": {"probe_copy_ms": ms_copy, "probe_copy_gbs": 2 * half / (ms_copy * 1e-3) / 1e9,
-                                                 "torch_copy_ms": ms_tcopy, "torch_copy_gbs": 2 * half / (ms_tcopy * 1e-3) / 1e9},
+                                                 "torch_copy_ms": ms_tcopy, "torch_copy_gbs": 2 * half / (ms_tcopy * 1e-3) / 1e9,
+                                                 "scattered_to_the_steps_pool_blocks_ms": ms_scopy,
+                                                 "scattered_to_the_steps_pool_blocks_gbs": 2 * half / (ms_scopy * 1e-3) / 1e9},
            "decode_shape": "7b/13b/30b, 56 tokens, three launches", "decode_ms": ms_d, "decode_bytes": bytes_d,
            "decode_gbs": bytes_d / (ms_d * 1e-3) / 1e9,
            "decode_one_fused_launch_ms": ms_d1, "decode_one_fused_launch_with_rope_ms": ms_dr,

@@ -202,6 +202,8 @@ def probe():
         lib.mux_probe_copy.argtypes = [c_vp, c_vp, c_i64, c_vp]
         lib.mux_probe_where.restype = c_i32
         lib.mux_probe_where.argtypes = [c_vp, c_i32, c_i32, c_vp]
+        lib.mux_probe_scatter_copy.restype = c_i32
+        lib.mux_probe_scatter_copy.argtypes = [c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_i64, c_vp]
         lib.mux_probe_mfma.restype = c_i32
         lib.mux_probe_mfma.argtypes = [c_i32] * 6 + [c_vp, c_vp, c_vp]
         _probe = lib

@@ -36,6 +36,14 @@ int32_t mux_probe_where(uint32_t *out, int32_t num_workgroups, int32_t spin_micr
  * yardstick for kernels that read and write equal amounts (the cache write). */
 int32_t mux_probe_copy(void *dst, const void *src, int64_t nbytes, void *stream);
 
+/* The same copy with the cache write's destinations: block b (4 KiB) of k_src
+ * and of v_src goes to pool block block_ids[b] (DEVICE int32 [n_blocks]; ids
+ * outside the pool are clamped) of k_pool and v_pool, read contiguously, written
+ * scattered - the byte movement of a prompt's cache write at block size 16
+ * without its windows, slot arithmetic and transposition. */
+int32_t mux_probe_scatter_copy(void *k_pool, void *v_pool, int64_t num_pool_blocks, const void *k_src,
+                               const void *v_src, const int32_t *block_ids, int64_t n_blocks, void *stream);
+
 /* What the matrix cores sustain: num_workgroups workgroups of
  * waves_per_workgroup (1..8) waves; waves below mfma_waves run `iterations`
  * iterations of `chains` (1, 2 or 4) independent v_mfma_f32_32x32x16_f16

@@ -129,6 +129,50 @@ extern "C" int32_t mux_probe_copy(void *dst, const void *src, int64_t nbytes, vo
 }
 
 // ---------------------------------------------------------------------------
+// The same copy with the cache write's destinations: the sources are read
+// contiguously, 4 KiB at a time, and every 4 KiB lands in the pool block the id
+// list names - one K block and one V block per workgroup, as the cache write of a
+// prompt leaves them, without its token windows, slot arithmetic and
+// transposition.  What separates this from the contiguous copy is the cost of
+// scattering the writes over the pool; what separates the cache write from this
+// is the cost of its own structure.
+// ---------------------------------------------------------------------------
+namespace mux {
+
+__global__ __launch_bounds__(256) void probe_scatter_copy_kernel(probe_u32x4 *__restrict__ k_dst,
+                                                                 probe_u32x4 *__restrict__ v_dst,
+                                                                 const probe_u32x4 *__restrict__ k_src,
+                                                                 const probe_u32x4 *__restrict__ v_src,
+                                                                 const int32_t *__restrict__ ids, int64_t num_pool_blocks) {
+  const int64_t b = blockIdx.x;
+  const int64_t last = num_pool_blocks - 1;
+  int64_t id = ids[b];
+  id = id < 0 ? 0 : (id > last ? last : id);               // ids outside the pool are clamped
+  const probe_u32x4 kx = __builtin_nontemporal_load(&k_src[b * 256 + threadIdx.x]);
+  const probe_u32x4 vx = __builtin_nontemporal_load(&v_src[b * 256 + threadIdx.x]);
+  __builtin_nontemporal_store(kx, &k_dst[id * 256 + threadIdx.x]);
+  __builtin_nontemporal_store(vx, &v_dst[id * 256 + threadIdx.x]);
+}
+
+}  // namespace mux
+
+extern "C" int32_t mux_probe_scatter_copy(void *k_pool, void *v_pool, int64_t num_pool_blocks, const void *k_src,
+                                          const void *v_src, const int32_t *block_ids, int64_t n_blocks, void *stream) {
+  if (!k_pool || !v_pool || !k_src || !v_src || num_pool_blocks <= 0 || n_blocks < 0) return -1;
+  if (n_blocks > 0 && !block_ids) return -1;
+  if ((reinterpret_cast<uintptr_t>(k_pool) | reinterpret_cast<uintptr_t>(v_pool) | reinterpret_cast<uintptr_t>(k_src) |
+       reinterpret_cast<uintptr_t>(v_src)) & 15u)
+    return -1;
+  if (n_blocks == 0) return 0;
+  if (n_blocks > 0x7fffffff) return -2;
+  hipLaunchKernelGGL(mux::probe_scatter_copy_kernel, dim3(static_cast<uint32_t>(n_blocks)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<mux::probe_u32x4 *>(k_pool),
+                     static_cast<mux::probe_u32x4 *>(v_pool), static_cast<const mux::probe_u32x4 *>(k_src),
+                     static_cast<const mux::probe_u32x4 *>(v_src), block_ids, num_pool_blocks);
+  return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
+// ---------------------------------------------------------------------------
 // What the matrix cores sustain, and what they sustain beside vector-ALU work:
 // waves 0 .. mfma_waves-1 of a workgroup run `iters` iterations of CHAINS
 // independent v_mfma_f32_32x32x16_f16 accumulations (operands in registers,

@@ -648,6 +648,67 @@ def test_gather_read_probe_runs_and_rejects_what_it_cannot_read():
                                              None) == -1      # invalid argument
 
 
+def test_copy_probe_copies_and_mfma_probe_reports_its_clocks():
+    """The two other yardsticks of bench.py: the contiguous copy (next to the
+    cache write) moves exactly the bytes it is given and refuses sizes and
+    pointers that are no multiple of its 16-byte chunk; the matrix-core loop
+    finishes, reports ticks of both clocks for every workgroup and refuses
+    combinations that were not built."""
+    print("[case] copy probe and mfma probe", flush=True)
+    from muxserve_amd import _lib
+    lib = _lib.probe()
+    st = torch.cuda.current_stream().cuda_stream
+    for n in (16, 4096, 16 * 257, 1 << 20):
+        src = torch.randint(0, 256, (n,), dtype=torch.uint8, device=DEV)
+        dst = torch.zeros(n + 32, dtype=torch.uint8, device=DEV)
+        assert lib.mux_probe_copy(dst.data_ptr(), src.data_ptr(), n, st) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(dst[:n], src) and int(dst[n:].sum()) == 0
+    src = torch.zeros(64, dtype=torch.uint8, device=DEV)
+    dst = torch.zeros(64, dtype=torch.uint8, device=DEV)
+    assert lib.mux_probe_copy(dst.data_ptr(), src.data_ptr(), 0, st) == 0
+    assert lib.mux_probe_copy(dst.data_ptr(), src.data_ptr(), 24, st) == -1
+    assert lib.mux_probe_copy(dst.data_ptr() + 4, src.data_ptr(), 32, st) == -1
+    assert lib.mux_probe_copy(None, src.data_ptr(), 32, st) == -1
+
+    # the copy with scattered destinations: block b of the sources lands in pool block ids[b]
+    N = 64
+    k_pool, v_pool = allocate_gpu_cache(N, 16, DEV)
+    k_pool.zero_()
+    v_pool.zero_()
+    ids = torch.tensor([5, 63, 0, 17, 99, -3], dtype=torch.int32, device=DEV)      # the last two are clamped to 63 and 0
+    ks = torch.randint(-30000, 30000, (ids.numel(), 2048), dtype=torch.int16, device=DEV)
+    vs = torch.randint(-30000, 30000, (ids.numel(), 2048), dtype=torch.int16, device=DEV)
+    assert lib.mux_probe_scatter_copy(k_pool.data_ptr(), v_pool.data_ptr(), N, ks.data_ptr(), vs.data_ptr(),
+                                      ids.data_ptr(), 4, st) == 0
+    torch.cuda.synchronize()
+    kp, vp = k_pool.view(torch.int16).view(N, 2048), v_pool.view(torch.int16).view(N, 2048)
+    for b, i in enumerate((5, 63, 0, 17)):
+        assert torch.equal(kp[i], ks[b]) and torch.equal(vp[i], vs[b])
+    untouched = [i for i in range(N) if i not in (5, 63, 0, 17)]
+    assert int(kp[untouched].abs().sum()) == 0 and int(vp[untouched].abs().sum()) == 0
+    assert lib.mux_probe_scatter_copy(k_pool.data_ptr(), v_pool.data_ptr(), N, ks.data_ptr(), vs.data_ptr(),
+                                      ids.data_ptr(), 6, st) == 0       # ids outside the pool: clamped, no stray write
+    assert lib.mux_probe_scatter_copy(k_pool.data_ptr(), v_pool.data_ptr(), 0, ks.data_ptr(), vs.data_ptr(),
+                                      ids.data_ptr(), 4, st) == -1
+    assert lib.mux_probe_scatter_copy(k_pool.data_ptr(), v_pool.data_ptr(), N, ks.data_ptr(), vs.data_ptr(),
+                                      None, 4, st) == -1
+    torch.cuda.synchronize()
+
+    sink = torch.zeros(1, dtype=torch.float32, device=DEV)
+    for chains, valu, waves, mfma_waves in ((1, 0, 4, 4), (4, 8, 4, 4), (4, 0, 8, 4), (2, 0, 1, 0)):
+        ticks = torch.zeros(8, 2, dtype=torch.int32, device=DEV)
+        assert lib.mux_probe_mfma(chains, valu, 200, 8, waves, mfma_waves, ticks.data_ptr(), sink.data_ptr(), st) == 0
+        torch.cuda.synchronize()
+        assert bool((ticks > 0).all())
+    ticks = torch.zeros(8, 2, dtype=torch.int32, device=DEV)
+    assert lib.mux_probe_mfma(3, 0, 200, 8, 4, 4, ticks.data_ptr(), sink.data_ptr(), st) == -2     # not built
+    assert lib.mux_probe_mfma(4, 0, 200, 8, 9, 4, ticks.data_ptr(), sink.data_ptr(), st) == -1
+    assert lib.mux_probe_mfma(4, 0, 0, 8, 4, 4, ticks.data_ptr(), sink.data_ptr(), st) == -1
+    torch.cuda.synchronize()
+    assert int(ticks.sum()) == 0
+
+
 def test_split_context_hand_off_is_stable_over_two_thousand_launches():
     """The hand-off of split contexts between workgroups (partial results
     published with device-coherent stores, one arrival counter per sequence and
