@@ -130,7 +130,16 @@ def test_colocated_prefill_and_decode_at_the_benchmark_shapes():
     pout = torch.zeros((T, Hp * D), dtype=torch.float16, device=DEV)
     s_prefill, s_decode = ops.CUMaskedStream(0, 40), ops.CUMaskedStream(40, 100)
     torch.cuda.synchronize()
-    for _ in range(3):
+    # Events at both ends of each stream's work, and one before all of it to measure from:
+    # the two shares of the GPU must really have been busy at the same time.
+    ev = {n: torch.cuda.Event(enable_timing=True) for n in ("t0", "p0", "p1", "d0", "d1")}
+    for rnd in range(4):
+        if rnd == 1:                    # the first round loads the kernels; the events bracket the other three
+            s_prefill.synchronize()
+            s_decode.synchronize()
+            ev["t0"].record()
+            ev["p0"].record(s_prefill.torch_stream)
+            ev["d0"].record(s_decode.torch_stream)
         with torch.cuda.stream(s_prefill.torch_stream):
             ops.prefill_causal(pout, q, k, v, cu, 1024, D ** -0.5, Hp)
             ops.reshape_and_cache(k, v, k_pool, v_pool, dslots)
@@ -139,8 +148,17 @@ def test_colocated_prefill_and_decode_at_the_benchmark_shapes():
                 ops.paged_decode(dec.out, dec.q, k_pool, v_pool, dec.d_block_tables, dec.d_context_lens,
                                  dec.max_context_len, dec.scale, total_context_len=int(ctx.sum()),
                                  context_lens_host=torch.from_numpy(ctx))
+    ev["p1"].record(s_prefill.torch_stream)
+    ev["d1"].record(s_decode.torch_stream)
     s_prefill.synchronize()
     s_decode.synchronize()
+    torch.cuda.synchronize()
+    at = {n: ev["t0"].elapsed_time(e) for n, e in ev.items() if n != "t0"}      # ms since t0
+    overlap = min(at["p1"], at["d1"]) - max(at["p0"], at["d0"])
+    shorter = min(at["p1"] - at["p0"], at["d1"] - at["d0"])
+    print(f"[colocated] prefill stream {at['p0']:.3f}..{at['p1']:.3f} ms, decode stream {at['d0']:.3f}..{at['d1']:.3f} ms, "
+          f"overlap {overlap:.3f} ms", flush=True)
+    assert overlap > 0.5 * shorter, (at, "the two streams did not run side by side")
     # prefill: heads 0, 17, 30, 51 of prompts 1 and 3 (causal attention is per head and per prompt)
     heads = [0, 17, 30, 51]
     cols = torch.cat([torch.arange(h * D, (h + 1) * D) for h in heads])
