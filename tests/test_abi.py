@@ -131,6 +131,58 @@ def test_workspace_size_does_not_depend_on_the_hint_and_host_pairs_are_exact():
             assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, partition) == (want if want <= 384 else 0)
 
 
+def test_library_chosen_partition_follows_the_size_of_the_launch():
+    """With partition_size 0 the library picks the partition: 256 tokens, but
+    1024 for one model's large batch (at least 1.5 M tokens x heads by the
+    caller's bound on the context sum, or by half the longest context per
+    sequence without one) and 512 beyond 4096-token contexts.  Seen through the
+    unit count of the host-side enumeration; the workspace asked for is never
+    smaller than what the 256-token partition needs, whichever is picked."""
+    import numpy as np
+    lib = _lib.attn()
+
+    def units(ctx, partition):
+        n = 0
+        for c in ctx:
+            fg, rem = divmod(int(c), partition)
+            n += fg + (1 if rem > 0 and not (fg > 0 and rem <= 16) else 0)
+        return n
+
+    def item(B, heads, ctx_value, hint):
+        ctx = np.full(B, ctx_value, dtype=np.int32)
+        it = _lib.MuxDecodeItem()
+        it.num_seqs, it.num_q_heads, it.num_kv_heads, it.num_layers = B, heads, heads, 1
+        it.max_context_len = ctx_value
+        it.max_blocks = (ctx_value + 15) // 16
+        it.total_context_len = hint
+        it.context_lens_host = ctx.ctypes.data
+        return it, ctx
+
+    # 128 sequences x 700 tokens x 32 heads = 2.9 M: long partitions, one unit per sequence
+    it, ctx = item(128, 32, 700, 128 * 700)
+    assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, 0) == units(ctx, 1024) == 128
+    big = lib.mux_paged_decode_workspace_bytes(ctypes.addressof(it), 1, 0)
+    assert big == lib.mux_paged_decode_workspace_bytes(ctypes.addressof(it), 1, 256)
+    assert big >= lib.mux_paged_decode_workspace_bytes(ctypes.addressof(it), 1, 1024)
+    # the same batch without the bound: 128 x 350 x 32 = 1.4 M, below the line
+    it, ctx = item(128, 32, 700, 0)
+    assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, 0) == units(ctx, 256) == 128 * 3
+    # a small batch keeps the short partitions
+    it, ctx = item(8, 32, 700, 8 * 700)
+    assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, 0) == units(ctx, 256) == 24
+    # two models in one launch keep them however large
+    pair = (_lib.MuxDecodeItem * 2)()
+    keep = []
+    for k in range(2):
+        one, c = item(64, 32, 700, 64 * 700)
+        keep.append(c)
+        pair[k] = one
+    assert lib.mux_paged_decode_host_pairs(ctypes.addressof(pair), 2, 0) == 2 * 64 * 3
+    # contexts beyond 4096 tokens: 512-token partitions for the vector-ALU kernel
+    it, ctx = item(4, 32, 5000, 4 * 5000)
+    assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, 0) == units(ctx, 512)
+
+
 # ---------------------------------------------------------------------------
 # Every entry point of include/muxserve_attn.h called once with well-formed
 # arguments.  No device is present where this runs, so nothing can be launched:

@@ -459,6 +459,23 @@ def test_multi_decode_mixed_head_groupings_and_a_large_batch_share_one_workspace
             _check(m.out[:m.batch].float().cpu(), want)
 
 
+@pytest.mark.parametrize("host_lens", [False, True])
+def test_decode_large_single_model_batch_takes_the_long_partitions(host_lens):
+    """One model's large batch (192 sequences of 600..1500 tokens, 8 heads: 1.6 M
+    tokens x heads by the caller's bound): the library picks 1024-token
+    partitions, waves walk several tiles, contexts beyond 1040 tokens are split
+    in two.  Against the oracle, and against the same batch with the 256-token
+    partitions of small launches."""
+    _announce(f"large single-model batch, host lens {host_lens}")
+    rng = np.random.Generator(np.random.PCG64(77))
+    ctx = rng.integers(600, 1501, size=192).astype(np.int32)
+    ctx[:4] = (1024, 1040, 1041, 1500)
+    got, want = _decode_case(78, ctx, 8, 8, 16, hint=True, host_lens=host_lens)
+    _check(got, want)
+    short, _ = _decode_case(78, ctx, 8, 8, 16, partition=256, hint=True, host_lens=host_lens)
+    assert (got - short).abs().max().item() <= 1e-3
+
+
 def test_decode_rejects_bad_arguments():
     _announce("decode argument validation")
     dk, dv = allocate_gpu_cache(8, 16, DEV)
