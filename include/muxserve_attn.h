@@ -112,8 +112,8 @@ int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t kv_row_strid
  * call is made, so leave this NULL for launches recorded into a HIP graph that
  * is replayed with changed lengths.  NULL = enumerate on the device.
  * partition_size: tokens per split of a context (multiple of 64), 0 = choose:
- * 256, or 1024 for a single model's large batch (at least 1.5 M tokens x head
- * groups by total_context_len, or by num_seqs * max_context_len / 2 without
+ * 256, or 1024 for a large launch (at least 1.5 M tokens x head groups over
+ * its models, by total_context_len or by num_seqs * max_context_len / 2 without
  * it), or 512 / 1024 when contexts exceed 4096 tokens.  The workspace size
  * reported for 0 covers every choice, so it may differ from launch to launch.
  * workspace: scratch for the partial results of split contexts and, for

@@ -1233,11 +1233,11 @@ int choose_partition(const MuxDecodeItem *items, int n_items, int requested) {
     token_heads += tokens * (it.num_q_heads / std::max(group, 1));
   }
   if (max_ctx > 4096) return all_grouped ? 1024 : 512;
-  // One model's large batch does better with long partitions (fewer units, hardly
-  // any hand-off: 2 - 6 % over batches of 0.8 - 1.7 GB); small launches and
-  // launches of several models need the many short units to fill the chip and
-  // to end evenly (1024-token partitions: +1 to +15 % there).
-  if (n_items == 1 && !all_grouped && token_heads >= 1500000) return 1024;
+  // A large launch does better with long partitions (fewer units, hardly any
+  // hand-off: 1 - 6 % over launches of 0.8 - 1.7 GB of K/V, one model or three);
+  // a small one needs the many short units to fill the chip and to end evenly
+  // (1024-token partitions: +1 to +15 % there).
+  if (!all_grouped && token_heads >= 1500000) return 1024;
   return 256;
 }
 

@@ -133,8 +133,8 @@ def test_workspace_size_does_not_depend_on_the_hint_and_host_pairs_are_exact():
 
 def test_library_chosen_partition_follows_the_size_of_the_launch():
     """With partition_size 0 the library picks the partition: 256 tokens, but
-    1024 for one model's large batch (at least 1.5 M tokens x heads by the
-    caller's bound on the context sum, or by half the longest context per
+    1024 for a large launch (at least 1.5 M tokens x heads over its models, by
+    the caller's bound on the context sum, or by half the longest context per
     sequence without one) and 512 beyond 4096-token contexts.  Seen through the
     unit count of the host-side enumeration; the workspace asked for is never
     smaller than what the 256-token partition needs, whichever is picked."""
@@ -170,13 +170,16 @@ def test_library_chosen_partition_follows_the_size_of_the_launch():
     # a small batch keeps the short partitions
     it, ctx = item(8, 32, 700, 8 * 700)
     assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, 0) == units(ctx, 256) == 24
-    # two models in one launch keep them however large
+    # the sizes of the models of one launch add up: 2 x (64 x 700 x 32) = 2.9 M
     pair = (_lib.MuxDecodeItem * 2)()
     keep = []
     for k in range(2):
         one, c = item(64, 32, 700, 64 * 700)
         keep.append(c)
         pair[k] = one
+    assert lib.mux_paged_decode_host_pairs(ctypes.addressof(pair), 2, 0) == 2 * 64
+    for k in range(2):
+        pair[k].total_context_len = 0          # 2 x (64 x 350 x 32) = 1.4 M
     assert lib.mux_paged_decode_host_pairs(ctypes.addressof(pair), 2, 0) == 2 * 64 * 3
     # contexts beyond 4096 tokens: 512-token partitions for the vector-ALU kernel
     it, ctx = item(4, 32, 5000, 4 * 5000)
