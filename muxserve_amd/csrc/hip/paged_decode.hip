@@ -1517,8 +1517,18 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
   char *ws = static_cast<char *>(workspace);
 
   // Items are launched in groups that share G (query heads per workgroup).
+  // Within a launch the items' workgroups follow each other, the item with the
+  // most sequences last: its many single-unit contexts, the cheapest units of the
+  // launch, are then what the launch ends with (the three-model mix over four
+  // sets of batches: 0.2 - 1.2 % faster than in the caller's order, which had the
+  // largest batch first; no result depends on the order).
+  int order[MUXA_MAX_DECODE_ITEMS];
+  for (int i = 0; i < n_items; ++i) order[i] = i;
+  std::stable_sort(order, order + n_items,
+                   [&](int a, int b) { return items[a].num_seqs < items[b].num_seqs; });
   bool done[MUXA_MAX_DECODE_ITEMS] = {false};
-  for (int first = 0; first < n_items; ++first) {
+  for (int of = 0; of < n_items; ++of) {
+    const int first = order[of];
     if (done[first]) continue;
     const int G = pick_group(items[first].num_q_heads / items[first].num_kv_heads);
     DecodeParams P = {};
@@ -1541,7 +1551,8 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
     bool host_pairs = true;
     {
       int n_pairs = 0;
-      for (int i = first; i < n_items && host_pairs; ++i) {
+      for (int oi = of; oi < n_items && host_pairs; ++oi) {
+        const int i = order[oi];
         const MuxDecodeItem &it = items[i];
         if (done[i] || pick_group(it.num_q_heads / it.num_kv_heads) != G) continue;
         if (it.num_seqs == 0 || it.max_context_len == 0) continue;
@@ -1556,7 +1567,8 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
     }
     int64_t work = 0;
     bool tightened = false;
-    for (int i = first; i < n_items; ++i) {
+    for (int oi = of; oi < n_items; ++oi) {
+      const int i = order[oi];
       if (done[i]) continue;
       const MuxDecodeItem &it = items[i];
       if (pick_group(it.num_q_heads / it.num_kv_heads) != G) continue;
