@@ -1325,7 +1325,7 @@ size_t plan_workspace(const MuxDecodeItem *items, int n_items, int partition, It
 // to out[*n]; false when they do not fit the kernel argument's table or its
 // 16-bit fields.
 bool enumerate_pairs_on_host(const int32_t *ctx_host, int B, int max_ctx, int partition, int rounds, int absorb,
-                             uint2 *out, int *n) {
+                             uint2 *out, int *n, int *first_single_out = nullptr) {
   if (B > 0xffff) return false;
   auto clamped = [&](int s) { return std::max(std::min(ctx_host[s], max_ctx), 0); };
   int at = *n;
@@ -1355,6 +1355,7 @@ bool enumerate_pairs_on_host(const int32_t *ctx_host, int B, int max_ctx, int pa
     if (c > 0 && seq_units(c, partition, rounds, absorb).count() == 1 && !push(s, 0, c)) return false;
   }
   std::stable_sort(out + first_single, out + at, [](const uint2 &a, const uint2 &b) { return a.y > b.y; });
+  if (first_single_out) *first_single_out = first_single;
   *n = at;
   return true;
 }
@@ -1548,6 +1549,7 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
     // Host-enumerated units: every item of the launch group must come with its
     // context lengths on the host, and the pairs must fit the kernel argument.
     int pair_begin[MUXA_MAX_DECODE_ITEMS] = {0}, pair_end[MUXA_MAX_DECODE_ITEMS] = {0};
+    int pair_single[MUXA_MAX_DECODE_ITEMS] = {0};          // the item's first single-unit context
     bool host_pairs = true;
     {
       int n_pairs = 0;
@@ -1559,7 +1561,7 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
         pair_begin[i] = n_pairs;
         host_pairs = it.context_lens_host != nullptr &&
                      enumerate_pairs_on_host(it.context_lens_host, it.num_seqs, it.max_context_len, partition,
-                                             rounds, absorb, P.pairs, &n_pairs);
+                                             rounds, absorb, P.pairs, &n_pairs, &pair_single[i]);
         pair_end[i] = n_pairs;
       }
       host_pairs = host_pairs && n_pairs > 0;
@@ -1567,15 +1569,10 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
     }
     int64_t work = 0;
     bool tightened = false;
-    for (int oi = of; oi < n_items; ++oi) {
-      const int i = order[oi];
-      if (done[i]) continue;
+    // What every descriptor of an item has in common.
+    auto describe = [&](DecodeItemDev &d, int i) {
       const MuxDecodeItem &it = items[i];
-      if (pick_group(it.num_q_heads / it.num_kv_heads) != G) continue;
-      done[i] = true;
-      if (it.num_seqs == 0 || it.max_context_len == 0) continue;
       const bool split = plan[i].max_splits > 1;
-      DecodeItemDev &d = P.it[P.n_items++];
       d.out = it.out;
       d.q = it.q;
       d.out_stride = it.out_row_stride;
@@ -1587,32 +1584,6 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
       d.ws_ml = split ? reinterpret_cast<float *>(ws + plan[i].ml_off) : nullptr;
       d.counters = split ? reinterpret_cast<int32_t *>(ws + plan[i].counters_off) : nullptr;
       d.unit_table = nullptr;
-      d.pair_begin = pair_begin[i];
-      if (host_pairs) {
-        // The grid holds exactly this item's pairs; no table, no padding.
-        d.B = it.num_seqs;
-        d.Hq = it.num_q_heads;
-        d.Hkv = it.num_kv_heads;
-        d.ratio = it.num_q_heads / it.num_kv_heads;
-        d.max_blocks = it.max_blocks;
-        d.max_splits = plan[i].max_splits;
-        d.max_ctx = it.max_context_len;
-        d.work_begin = static_cast<int32_t>(work);
-        d.scale_log2 = it.scale * 1.4426950408889634f;
-        work += static_cast<int64_t>(pair_end[i] - pair_begin[i]) * (it.num_q_heads / G);
-        continue;
-      }
-      if (plan[i].table_off != 0) {
-        const int64_t rows = static_cast<int64_t>(it.num_seqs) * plan[i].max_splits;
-        if (rows > 0x7fffffff) return MUXA_EUNSUPPORTED;
-        PlanItem &t = PP.it[n_tables++];
-        t.ctx = it.context_lens;
-        t.table = reinterpret_cast<int4 *>(ws + plan[i].table_off);
-        t.B = it.num_seqs;
-        t.max_ctx = it.max_context_len;
-        t.capacity = static_cast<int32_t>(rows);
-        d.unit_table = t.table;
-      }
       d.B = it.num_seqs;
       d.Hq = it.num_q_heads;
       d.Hkv = it.num_kv_heads;
@@ -1620,13 +1591,61 @@ int32_t multi_decode_impl(const MuxDecodeItem *items, int32_t n_items,
       d.max_blocks = it.max_blocks;
       d.max_splits = plan[i].max_splits;
       d.max_ctx = it.max_context_len;
-      d.work_begin = static_cast<int32_t>(work);
       d.scale_log2 = it.scale * 1.4426950408889634f;
-      if (plan[i].units > 0x7fffffff) return MUXA_EUNSUPPORTED;
-      d.pair_begin = static_cast<int32_t>(plan[i].units);       // pairs with a place in the grid
-      if (plan[i].units < static_cast<int64_t>(it.num_seqs) * plan[i].max_splits) tightened = true;
-      work += plan[i].units * (it.num_q_heads / G);
-      if (work > 0x7fffffff) return MUXA_EUNSUPPORTED;
+    };
+    int members[MUXA_MAX_DECODE_ITEMS], n_members = 0;
+    for (int oi = of; oi < n_items; ++oi) {
+      const int i = order[oi];
+      if (done[i]) continue;
+      const MuxDecodeItem &it = items[i];
+      if (pick_group(it.num_q_heads / it.num_kv_heads) != G) continue;
+      done[i] = true;
+      if (it.num_seqs == 0 || it.max_context_len == 0) continue;
+      members[n_members++] = i;
+    }
+    if (host_pairs) {
+      // The grid holds exactly the enumerated pairs; no table, no padding.  A
+      // descriptor is a run of pairs of one model; with room for two per model the
+      // units of split contexts of ALL models come first and the single-unit
+      // contexts of all models after them, so that the launch as a whole - not each
+      // model's stretch of it - ends with its cheapest units.
+      const bool two_runs = 2 * n_members <= MUXA_MAX_DECODE_ITEMS;
+      for (int pass = 0; pass < (two_runs ? 2 : 1); ++pass)
+        for (int m = 0; m < n_members; ++m) {
+          const int i = members[m];
+          const int lo = two_runs && pass == 1 ? pair_single[i] : pair_begin[i];
+          const int hi = two_runs && pass == 0 ? pair_single[i] : pair_end[i];
+          if (hi <= lo) continue;
+          DecodeItemDev &d = P.it[P.n_items++];
+          describe(d, i);
+          d.pair_begin = lo;
+          d.work_begin = static_cast<int32_t>(work);
+          work += static_cast<int64_t>(hi - lo) * (items[i].num_q_heads / G);
+        }
+    } else {
+      for (int m = 0; m < n_members; ++m) {
+        const int i = members[m];
+        const MuxDecodeItem &it = items[i];
+        DecodeItemDev &d = P.it[P.n_items++];
+        describe(d, i);
+        if (plan[i].table_off != 0) {
+          const int64_t rows = static_cast<int64_t>(it.num_seqs) * plan[i].max_splits;
+          if (rows > 0x7fffffff) return MUXA_EUNSUPPORTED;
+          PlanItem &t = PP.it[n_tables++];
+          t.ctx = it.context_lens;
+          t.table = reinterpret_cast<int4 *>(ws + plan[i].table_off);
+          t.B = it.num_seqs;
+          t.max_ctx = it.max_context_len;
+          t.capacity = static_cast<int32_t>(rows);
+          d.unit_table = t.table;
+        }
+        d.work_begin = static_cast<int32_t>(work);
+        if (plan[i].units > 0x7fffffff) return MUXA_EUNSUPPORTED;
+        d.pair_begin = static_cast<int32_t>(plan[i].units);       // pairs with a place in the grid
+        if (plan[i].units < static_cast<int64_t>(it.num_seqs) * plan[i].max_splits) tightened = true;
+        work += plan[i].units * (it.num_q_heads / G);
+        if (work > 0x7fffffff) return MUXA_EUNSUPPORTED;
+      }
     }
     if (P.n_items == 0) continue;
     if (n_tables > 0) {
