@@ -423,6 +423,64 @@ def test_multi_decode_three_models_one_launch_matches_separate_launches():
         _check(f[:m.batch].float().cpu(), want)
 
 
+@pytest.mark.parametrize("n_models", [2, 4, 5, 8])
+def test_multi_decode_layout_of_the_launch_changes_no_result(n_models):
+    """Inside a fused launch the library lays the models out by sequence count and,
+    with units enumerated on the host and at most four models, in two runs per
+    model (units of split contexts of all models, then all single-unit contexts);
+    with five to eight models each keeps one run.  Whatever the layout, every
+    model's output is bitwise what its own launch gives - models with only
+    single-unit contexts, only split contexts, one sequence, and equal sequence
+    counts included."""
+    _announce(f"multi decode layout, {n_models} models")
+    bs, N = 16, 40000
+    rng = np.random.Generator(np.random.PCG64(300 + n_models))
+    ids = rng.permutation(N)
+    kinds = [lambda: rng.integers(1, 900, size=9),          # mixed
+             lambda: rng.integers(1, 257, size=12),         # single-unit contexts only
+             lambda: rng.integers(300, 1200, size=5),       # split contexts only
+             lambda: rng.integers(1, 700, size=1),          # one sequence
+             lambda: rng.integers(1, 900, size=9),          # as many sequences as the first
+             lambda: rng.integers(1, 600, size=3),
+             lambda: rng.integers(200, 800, size=7),
+             lambda: rng.integers(1, 300, size=16)]
+    heads = [4, 2, 3, 5, 1, 2, 4, 3]
+    models, cur = [], 0
+    for k in range(n_models):
+        ctx = kinds[k]().astype(np.int32)
+        bt, cur = workloads.build_tables(ctx, heads[k], bs, ids, cur)
+        models.append(workloads.DecodeModel(f"m{k}", heads[k], heads[k], ctx, bt))
+    dk, dv = allocate_gpu_cache(N, bs, DEV)
+    dk.fill_(float("nan"))
+    dv.fill_(float("nan"))
+    workloads.fill_blocks(dk, dv, np.concatenate([m.used_blocks(bs) for m in models]), seed=5)
+    for i, m in enumerate(models):
+        m.to_device(DEV, torch.float16, seed=40 + i)
+    separate = []
+    for m in models:
+        m.out.zero_()
+        ops.paged_decode(m.out, m.q, dk, dv, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                         partition_size=256)
+        torch.cuda.synchronize()
+        separate.append(m.out.clone())
+    for host in (True, False):
+        calls = [ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                                total_context_len=int(m.context_lens.sum()),
+                                context_lens_host=torch.from_numpy(np.ascontiguousarray(m.context_lens, dtype=np.int32))
+                                if host else None) for m in models]
+        for rep in range(2):            # twice: the arrival counters must come back to zero
+            for m in models:
+                m.out.zero_()
+            ops.multi_decode(calls, dk, dv, partition_size=256)
+            torch.cuda.synchronize()
+            for m, sep in zip(models, separate):
+                assert torch.equal(m.out, sep), (m.name, host, rep)
+    ks, vs, tables = workloads.compact_to_host(dk, dv, models[:2], bs)
+    for m, t in zip(models[:2], tables):
+        want = orc.paged_decode(m.q.cpu(), ks, vs, t, m.context_lens, m.scale)
+        _check(m.out[:m.batch].float().cpu(), want)
+
+
 def test_multi_decode_mixed_head_groupings_and_a_large_batch_share_one_workspace():
     """One call with a grouped-query model (matrix-core kernel), a small
     multi-head model (register lookup) and a 300-sequence multi-head model
