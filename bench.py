@@ -50,6 +50,9 @@ def parse():
     ap.add_argument("--sets", type=int, default=6, help="distinct batches rotated through")
     ap.add_argument("--partition", type=int, default=0, help="tokens per context split (0 = library default)")
     ap.add_argument("--pool-util", type=float, default=0.6)
+    ap.add_argument("--batch-scale", type=int, default=1,
+                    help="mixed3_decode: multiply the three models' batches (32/16/8 sequences) by this; 1 is the "
+                         "headline configuration, larger values show how the launch scales")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-hint", action="store_true", help="do not pass the host-side sum of context lengths")
@@ -853,12 +856,17 @@ def main():
 
     # Disjoint ids for all sets from one seeded draw over the whole pool.
     rng = np.random.Generator(np.random.PCG64(args.seed))
-    probe = [workloads.config2(seed=args.seed + 1 + i, num_pool_blocks=N, id_perm=np.arange(1 << 20))[1]
+    if args.batch_scale < 1 or args.batch_scale > 8:
+        raise SystemExit("--batch-scale takes 1..8")
+    batches = tuple(b * args.batch_scale for b in (32, 16, 8))
+    probe = [workloads.config2(seed=args.seed + 1 + i, num_pool_blocks=N, id_perm=np.arange(1 << 23),
+                               batches=batches)[1]
              for i in range(args.sets)]
     ids = rng.choice(N, size=int(sum(probe)), replace=False)
     sets, off = [], 0
     for i in range(args.sets):
-        models, need = workloads.config2(seed=args.seed + 1 + i, num_pool_blocks=N, id_perm=ids[off:off + probe[i]])
+        models, need = workloads.config2(seed=args.seed + 1 + i, num_pool_blocks=N, id_perm=ids[off:off + probe[i]],
+                                         batches=batches)
         off += need
         used = np.concatenate([m.used_blocks(bs) for m in models])
         workloads.fill_blocks(k_pool, v_pool, used, seed=args.seed + 100 + i)
@@ -942,7 +950,8 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "mixed3_decode",
-            "models": "7b(H32,B32)+13b(H40,B16)+30b(H52,B8), one layer each, one fused launch per step",
+            "models": f"7b(H32,B{batches[0]})+13b(H40,B{batches[1]})+30b(H52,B{batches[2]}), one layer each, "
+                      "one fused launch per step",
             "head_size": 128, "block_size": bs, "pool_blocks": int(N), "pool_gb": round(N * 8192 / 1e9, 1),
             "tokens_per_step": tokens, "sets": args.sets, "partition": args.partition,
             "bytes_per_step": int(avg_bytes), "fused": not args.unfused, "seed": args.seed,
