@@ -1339,6 +1339,13 @@ bool enumerate_pairs_on_host(const int32_t *ctx_host, int B, int max_ctx, int pa
     const SeqUnits su = seq_units(c, partition, rounds, absorb);
     if (su.count() > 1 && su.rem > 0 && !push(s, su.nb, c)) return false;
   }
+  // (the remainders longest first: the same units, in the order that leaves the
+  // short ones for when the others are under way; long-context grouped-query
+  // batches 0.8 % faster, the three-model mix -0.7 to +0.2 us)
+  {
+    const uint32_t P = static_cast<uint32_t>(partition);
+    std::stable_sort(out + *n, out + at, [P](const uint2 &a, const uint2 &b) { return a.y % P > b.y % P; });
+  }
   for (int s = 0; s < B; ++s) {
     const int c = clamped(s);
     const SeqUnits su = seq_units(c, partition, rounds, absorb);
