@@ -63,9 +63,13 @@ def parse():
     ap.add_argument("--no-prompt-lens", action="store_true",
                     help="prefill3: do not pass the host-side prompt lengths (grid sized by the longest prompt)")
     ap.add_argument("--unfused", action="store_true", help="one launch per model instead of one fused launch")
+    ap.add_argument("--prompt-cap", type=int, default=0,
+                    help="prefill_timeline: cut the prompts of the three-model mix at this length (0 = as drawn)")
+    ap.add_argument("--long-prompts", action="store_true",
+                    help="prefill_timeline: 16 prompts of 2048 tokens, 32 heads, instead of the three-model mix")
     ap.add_argument("--workload", default="mixed3_decode",
                     choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long", "model_ops", "host_step",
-                             "cu_masks", "prefill_long", "decode_timeline", "mfma_ceiling"],
+                             "cu_masks", "prefill_long", "decode_timeline", "prefill_timeline", "mfma_ceiling"],
                     help="mixed3_decode is the headline metric; the others are the remaining synthetic "
                          "shapes, each printing its own JSON line")
     return ap.parse_args()
@@ -130,6 +134,12 @@ def _time(fn, steps, warmup, stream=None):
     return e0.elapsed_time(e1) / steps
 
 
+# The matrix-core kernels of a process start below their later rate: the first tens of launches run at a lower
+# shader clock (SQ_BUSY_CU_CYCLES per launch stays the same while the launch takes up to a fifth longer).  The prefill
+# workloads therefore warm up with at least this many launches and report the first launches' time beside the steady one.
+PREFILL_MIN_WARMUP = 100
+
+
 def _line(metric, value, unit, args, ms, config, roofline, dtype="f16", higher=True):
     return {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": higher, "scaling": "weak",
@@ -178,19 +188,23 @@ def bench_prefill3(args):
         for m, q, k, v, out, cu, slots, T, order in work:
             ops.reshape_and_cache(k, v, k_pool, v_pool, slots, num_tokens=T)
 
-    ms_separate = _time(attn, args.steps, args.warmup)
     # the three models' prompts in ONE launch, and the three cache writes in one
     pcalls = [ops.PrefillCall(out, q, k, v, cu, [int(x) for x in m.prompt_lens], m.scale, m.num_kv_heads)
               for m, q, k, v, out, cu, slots, T, order in work]
     wcalls = [ops.CacheWriteCall(k, v, slots, num_tokens=T) for m, q, k, v, out, cu, slots, T, order in work]
-    ms_a = ms_separate if args.unfused else _time(lambda _: ops.multi_prefill_causal(pcalls), args.steps, args.warmup)
+    fused = (lambda _: ops.multi_prefill_causal(pcalls)) if not args.unfused else attn
+    ms_first = _time(fused, 20, 0)
+    warm = max(args.warmup, PREFILL_MIN_WARMUP)
+    ms_separate = _time(attn, args.steps, warm)
+    ms_a = ms_separate if args.unfused else _time(fused, args.steps, warm)
     ms_w_separate = _time(write, args.steps, args.warmup)
     ms_w = ms_w_separate if args.unfused else _time(lambda _: ops.multi_reshape_and_cache(wcalls, k_pool, v_pool),
                                                     args.steps, args.warmup)
     tf = flops / (ms_a * 1e-3) / 1e12
     gbs = wbytes / (ms_w * 1e-3) / 1e9
     cfg = {"workload": "prefill3", "prompts_per_model": 16, "tokens": tokens, "flops": flops,
-           "fused": not args.unfused, "one_launch_per_model_ms": ms_separate,
+           "fused": not args.unfused, "one_launch_per_model_ms": ms_separate, "warmup_launches": warm,
+           "first_20_launches_of_the_process_ms": ms_first,
            "cache_write_one_launch_per_model_ms": ms_w_separate, "cache_write_ms": ms_w, "cache_write_gbs": gbs, "cache_write_frac_of_hbm": gbs / HBM_PEAK_GBS}
     roof = {"bound": "mfma", "achieved": tf, "peak": 2500.0, "unit": "TFLOP/s", "frac": tf / 2500.0,
             "traffic": None, "kernel": "prefill_causal_kernel<F16>"}
@@ -211,11 +225,15 @@ def bench_prefill_long(args):
     out = torch.empty((P * L, H * D), dtype=torch.float16, device=dev)
     cu = torch.arange(0, P * L + 1, L, dtype=torch.int32, device=dev)
     lens = [L] * P
-    ms = _time(lambda _: ops.prefill_causal(out, q, k, v, cu, L, D ** -0.5, H,
-                                            prompt_lens=None if args.no_prompt_lens else lens), args.steps, args.warmup)
+    step = lambda _: ops.prefill_causal(out, q, k, v, cu, L, D ** -0.5, H,                          # noqa: E731
+                                        prompt_lens=None if args.no_prompt_lens else lens)
+    ms_first = _time(step, 20, 0)
+    warm = max(args.warmup, PREFILL_MIN_WARMUP)
+    ms = _time(step, args.steps, warm)
     flops = workloads.prefill_flops(np.asarray(lens), H)
     tf = flops / (ms * 1e-3) / 1e12
-    cfg = {"workload": "prefill_long", "prompts": P, "prompt_len": L, "heads": H, "flops": flops}
+    cfg = {"workload": "prefill_long", "prompts": P, "prompt_len": L, "heads": H, "flops": flops,
+           "warmup_launches": 20 + warm, "first_20_launches_of_the_process_ms": ms_first}
     roof = {"bound": "mfma", "achieved": tf, "peak": 2500.0, "unit": "TFLOP/s", "frac": tf / 2500.0,
             "traffic": None, "kernel": "prefill_causal_kernel<F16>"}
     return _line("prefill causal attention tokens/s (16 prompts x 2048 tokens, 32 heads)", P * L / (ms * 1e-3),
@@ -562,6 +580,108 @@ def bench_decode_timeline(args):
                   "kernel": "paged_decode_kernel<F16,16,1,4> with phase stamps"}, higher=False)
 
 
+def bench_prefill_timeline(args):
+    """Workgroup timeline of one launch of the prefill kernel, from the tracing
+    build of the library (libmuxattn_trace.so): thread 0 of every workgroup
+    stamps the 100 MHz clock at its entry, when the prompt's offsets are known,
+    when its first key tile has landed, after its last key tile and after
+    issuing its output stores.  Default: the three
+    models' 16 prompts each in one launch (--prompt-cap N cuts them at N
+    tokens); --long-prompts: 16 x 2048 tokens, 32 heads."""
+    import ctypes
+    import torch
+    from muxserve_amd import _lib, ops, workloads
+    from muxserve_amd.build import TRACE_LIB
+    from muxserve_amd.pool import HEAD_SIZE as D
+    if os.path.abspath(_lib.ATTN_LIB_PATH) != os.path.abspath(TRACE_LIB):
+        raise SystemExit("prefill_timeline needs the tracing build: python -m muxserve_amd.build trace, then run with "
+                         f"MUXSERVE_ATTN_LIB={TRACE_LIB}")
+    lib = _lib.attn()
+    lib.mux_prefill_trace_set.restype = ctypes.c_int32
+    lib.mux_prefill_trace_set.argtypes = [ctypes.c_void_p, ctypes.c_int64]
+    dev = "cuda:0"
+    if args.long_prompts:
+        models = [workloads.PrefillModel("7b", 32, 32, np.full(16, 2048, dtype=np.int64))]
+    else:
+        models = workloads.config3(seed=args.seed)
+        if args.prompt_cap > 0:
+            for m in models:
+                m.prompt_lens = np.minimum(m.prompt_lens, args.prompt_cap)
+    g = torch.Generator().manual_seed(args.seed)
+    calls, flops = [], 0.0
+    for m in models:
+        T, Hq, Hkv = m.num_tokens, m.num_q_heads, m.num_kv_heads
+        pad = (T + 7) // 8 * 8
+        qkv = torch.randn((pad, (Hq + 2 * Hkv) * D), generator=g).half().to(dev)
+        q, k, v = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+        out = torch.empty((pad, Hq * D), dtype=torch.float16, device=dev)
+        cu = torch.from_numpy(m.cu_seqlens()).to(dev)
+        calls.append(ops.PrefillCall(out, q, k, v, cu, [int(x) for x in m.prompt_lens], m.scale, Hkv))
+        flops += workloads.prefill_flops(m.prompt_lens, Hq)
+    rows = 16384
+    table = torch.zeros((rows, 8), dtype=torch.int64, device=dev)
+    # What the stamps cost: the launches with the table switched off and on, after the warm-up.
+    ms_off = _time(lambda _: ops.multi_prefill_causal(calls), 30, max(args.warmup, 150))
+    assert lib.mux_prefill_trace_set(table.data_ptr(), rows) == 0
+    ms_on = _time(lambda _: ops.multi_prefill_causal(calls), 30, 5)
+    # Every launch stamps the same rows, so after a run of back-to-back launches the table holds
+    # the last one's - a launch in the middle of a busy stream, as in the benchmark loop.
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    # (the first tens of launches of a process run up to a fifth slower than the later ones)
+    for _ in range(20):
+        ops.multi_prefill_causal(calls)
+    e0.record()
+    ops.multi_prefill_causal(calls)
+    e1.record()
+    torch.cuda.synchronize()
+    lib.mux_prefill_trace_set(None, 0)
+    t = table.cpu().numpy()
+    t = t[t[:, 0] > 0]
+    base = t[:, 0].min()
+    us = lambda x: (x - base) / 100.0                                                   # noqa: E731
+    a, known, b, c, d = (us(t[:, i]) for i in range(5))
+    nt, plen, q0 = t[:, 5], t[:, 6], t[:, 7]
+    span, life = float(d.max()), d - a
+    slots = 3 * torch.cuda.get_device_properties(0).multi_processor_count
+    # 32 x 32 score blocks the waves of a workgroup really compute (a wave skips the tiles in
+    # its rows' future and rows past the prompt's end), against the causal triangle's share
+    rows_left = np.clip(plen - q0, 0, 128)
+    waves = (rows_left + 31) // 32
+    blocks_done = sum(int(((q0 // 32 + w + 1) * (waves > w)).sum()) for w in range(4))
+    blocks_ideal = float(sum(((q0[i] + np.arange(rows_left[i]) + 1).sum()) for i in range(len(t)))) / 1024.0
+    by_tiles = []
+    for lo, hi in ((1, 2), (2, 4), (4, 8), (8, 16), (16, 32), (32, 65)):
+        m = (nt >= lo) & (nt < hi)
+        if m.any():
+            by_tiles.append({"key_tiles": f"{lo}..{hi - 1}", "workgroups": int(m.sum()), "life_us": float(life[m].mean()),
+                             "prologue_us": float((b - a)[m].mean()),
+                             "us_per_key_tile": float((c - b)[m].sum() / nt[m].sum()),
+                             "epilogue_us": float((d - c)[m].mean())})
+    bins, step = [], max(2.0, round(span / 24.0))
+    for lo in np.arange(0.0, span + step, step):
+        mid = lo + step / 2
+        bins.append({"t_us": float(lo), "resident": int(((a <= mid) & (d > mid)).sum()),
+                     "in_tile_loop": int(((b <= mid) & (c > mid)).sum())})
+    cfg = {"workload": "prefill_timeline", "prompts": "16 x 2048, 32 heads" if args.long_prompts else
+           f"three models x 16 prompts, cap {args.prompt_cap or None}", "flops": flops,
+           "kernel_ms_with_stamps": e0.elapsed_time(e1), "ms_per_launch_table_off": ms_off,
+           "ms_per_launch_table_on": ms_on, "span_us": span, "workgroups_with_work": int(len(t)),
+           "workgroup_slots": int(slots), "slot_time_filled": float(life.sum() / (span * slots)),
+           "share_of_workgroup_life": {"prologue": float((b - a).sum() / life.sum()),
+                                       "tile_loop": float((c - b).sum() / life.sum()),
+                                       "epilogue": float((d - c).sum() / life.sum())},
+           "mean_us": {"prologue": float((b - a).mean()), "of_it_until_the_prompt_is_known": float((known - a).mean()),
+                       "per_key_tile": float((c - b).sum() / nt.sum()),
+                       "epilogue": float((d - c).mean()), "life": float(life.mean())},
+           "key_tiles_per_workgroup": float(nt.mean()),
+           "score_blocks_32x32": {"computed": int(blocks_done), "causal_triangle": blocks_ideal,
+                                  "useful_fraction": blocks_ideal / blocks_done},
+           "last_start_us": float(a.max()), "by_key_tiles": by_tiles, "bins": bins}
+    return _line("prefill kernel workgroup timeline (tracing build)", span, "us", args, span * 1e-3, cfg,
+                 {"bound": "mfma", "achieved": None, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": None,
+                  "traffic": None, "kernel": "prefill_causal_kernel<F16> with workgroup stamps"}, higher=False)
+
+
 def bench_gqa_long(args):
     """Config 5: 64 query heads over 8 kv heads, bf16, batch 64, ctx U[2048, 8192]."""
     import torch
@@ -838,6 +958,7 @@ def main():
               file=sys.stderr)
         sys.exit(2)
     other = {"prefill3": bench_prefill3, "cache_write": bench_cache_write, "colocated": bench_colocated, "cu_masks": bench_cu_masks, "prefill_long": bench_prefill_long, "decode_timeline": bench_decode_timeline,
+             "prefill_timeline": bench_prefill_timeline,
              "gqa_long": bench_gqa_long, "model_ops": bench_model_ops, "host_step": bench_host_step,
              "mfma_ceiling": bench_mfma_ceiling}
     if args.workload in other:

@@ -41,6 +41,18 @@ constexpr int kNKB = kBN / 32;           // 32-key blocks (one MFMA row block) p
 // Query tiles listed in the kernel argument (its size limit is 4 KiB).
 constexpr int kMaxPairs = 768;
 
+// Tracing build (-DMUX_TRACE, libmuxattn_trace.so; never the shipped library):
+// thread 0 of every workgroup that has work stamps the 100 MHz clock into a
+// caller-provided table, 8 int64 per workgroup: [0] entry, [1] the prompt's
+// place and length known, [2] first key tile landed and the workgroup met (end
+// of the prologue), [3] last key tile done, [4] output stores issued (a wave
+// does not wait for them before it ends, and neither does the stamp), [5] key
+// tiles of the workgroup, [6] prompt length, [7] first query row.
+#ifdef MUX_TRACE
+__device__ long long *g_prefill_trace = nullptr;
+__device__ long long g_prefill_trace_rows = 0;
+#endif
+
 union Frag {
   u32x4 u;
   v8f16 h;
@@ -137,6 +149,12 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
   constexpr int kSmemElems = 4 * kTileElems > 4 * 32 * (D + 8) ? 4 * kTileElems : 4 * 32 * (D + 8);
   __shared__ __attribute__((aligned(16))) uint16_t smem[kSmemElems];
 
+#ifdef MUX_TRACE
+  const long long tr_entry = __builtin_amdgcn_s_memrealtime();
+  long long tr_first = 0;
+  long long *const tr_table = g_prefill_trace;   // read here, so that the write at the end waits for nothing
+  const long long tr_rows = g_prefill_trace_rows;
+#endif
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -183,6 +201,10 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
   const int seq_begin = I.cu_seqlens[prompt];
   const int len = I.cu_seqlens[prompt + 1] - seq_begin;
   if (q0 >= len) return;
+#ifdef MUX_TRACE
+  asm volatile("s_nop 0" ::"s"(len));    // (the stamp waits for the loads of the two offsets)
+  const long long tr_len = __builtin_amdgcn_s_memrealtime();
+#endif
 
   const int qcol = lane & 31;            // this lane's query column / fragment row
   const int half = lane >> 5;            // which 8 of a fragment's 16 k-slots
@@ -260,6 +282,9 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
     // and everybody is done with the other buffer.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+#ifdef MUX_TRACE
+    if (t == 0) tr_first = __builtin_amdgcn_s_memrealtime();
+#endif
     if (t + 1 < n_tiles) dma_tile(cur ^ 1);
     // Nothing to compute: every key of the tile is in this wave's future, or all
     // of the wave's rows are past the prompt's end.
@@ -419,6 +444,9 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
     }
   }
 
+#ifdef MUX_TRACE
+  const long long tr_loop = __builtin_amdgcn_s_memrealtime();
+#endif
   // ---- normalise and store: register i of block mb is d = 32 mb + 8 (i/4) + 4 half + i%4 ------
   const float l_tot = sum_with_lane_xor32(l_run);
   const float inv = 1.f / l_tot;
@@ -461,6 +489,13 @@ __global__ __launch_bounds__(256, 3) void prefill_causal_kernel(const PrefillPar
         *reinterpret_cast<uint2 *>(op + 32 * mb + 8 * g) = w2;
       }
   }
+#ifdef MUX_TRACE
+  if (tid == 0 && tr_table && blockIdx.x < tr_rows) {
+    long long *row = tr_table + 8 * static_cast<long long>(blockIdx.x);
+    row[0] = tr_entry, row[1] = tr_len, row[2] = tr_first, row[3] = tr_loop, row[4] = __builtin_amdgcn_s_memrealtime();
+    row[5] = n_tiles, row[6] = len, row[7] = q0;
+  }
+#endif
 }
 
 }  // namespace mux
@@ -650,3 +685,15 @@ extern "C" int32_t mux_prefill_causal(void *out, int64_t out_row_stride, const v
   if (launch_compact(&it, 1, dtype, st, &rc)) return rc;
   return launch_dense(it, prompt_order, dtype, st);
 }
+
+#ifdef MUX_TRACE
+// Tracing build only: where the prefill kernel's workgroups write their stamps
+// (DEVICE int64 [rows, 8], zero-filled by the caller; NULL switches it off).
+extern "C" int32_t mux_prefill_trace_set(void *table, int64_t rows) {
+  long long *p = static_cast<long long *>(table);
+  long long n = table ? rows : 0;
+  MUX_HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(mux::g_prefill_trace), &p, sizeof(p)));
+  MUX_HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(mux::g_prefill_trace_rows), &n, sizeof(n)));
+  return MUXA_OK;
+}
+#endif
