@@ -44,12 +44,16 @@ def main():
     while not ask("start_warmup"):            # one runtime warms up at a time (llm_runtime.py:600-640)
         time.sleep(0.01)
     ask("warmup_ready")
+    while not ask("init_finished"):           # serve only once every runtime is up, so that the runtimes' steps interleave
+        time.sleep(0.005)
 
     bs, max_seq = 16, 512
     rng = np.random.Generator(np.random.PCG64(seed))
     sched = BatchScheduler(L, H, max_seq, bs)
     alloc = lambda r: ask("cache_alloc", [model, r])      # noqa: E731
-    next_id = 0
+    # Request ids are unique across the models of a FlexStore: its one KVStorage keys the blocks by
+    # request id alone (muxserve/flexstore/manager.py:776-790; the scheduler hands out global ids).
+    next_id = 1000 * seed
     live = []
     steps_done = []
     for wave in range(3):
