@@ -50,7 +50,12 @@ int64_t mux_kvstorage_allocate_batch_bound(const int32_t *info, int32_t n_info,
 /* KVStorage::allocateBatch, csrc/memory_manager.cpp:25-142.  info is
  * int32[n_info] = rows (request id, token blocks wanted, prompt-allocated
  * flag).  Writes [preemptIdx, ids...] to out and returns its length
- * (1 when preemptIdx <= 0).  MUX_ENOSPC if out_cap is too small. */
+ * (1 when preemptIdx <= 0).  MUX_ENOSPC if out_cap is too small.  The blocks
+ * are keyed by request id alone, whatever the (num_layers, num_heads) of the
+ * call: callers that share one KVStorage - the models of a FlexStore - must
+ * hand out ids that are unique among them.  A row that asks for fewer blocks
+ * than its id already holds (the sign of two callers using one id) returns
+ * MUX_ESTATE where the reference asserts or copies from before the list. */
 int64_t mux_kvstorage_allocate_batch(MuxKVStorage *s, const int32_t *info, int32_t n_info,
                                      int32_t num_layers, int32_t num_heads,
                                      int32_t *out, int64_t out_cap);
