@@ -1048,6 +1048,12 @@ def main():
                      args.steps, args.warmup)
     probe_bytes = sum(int(s[2].numel()) * 8192 * v for s, v in
                       zip(sets, [len(range(i, args.steps, len(sets))) for i in range(len(sets))])) / args.steps
+    # And what the chip reads at all in a launch of this size: the same probe over as many blocks
+    # in one consecutive run of the pool (a different run per batch, far apart).
+    runs = [torch.arange(int(s[2].numel()), dtype=torch.int32, device=dev) + int(i * (N // len(sets)))
+            for i, s in enumerate(sets)]
+    run_ms = _time(lambda i: workloads.probe_gather_read(k_pool, v_pool, runs[i % len(runs)], sink),
+                   args.steps, args.warmup)
 
     tokens = sum(m.batch for m in sets[0][0])
     step_bytes = [sum(workloads.decode_bytes(m.context_lens, m.num_q_heads, m.num_kv_heads, bs) for m in models)
@@ -1095,6 +1101,8 @@ def main():
             "bare_gather_read_of_the_same_blocks": {
                 "ms": probe_ms, "bytes": int(probe_bytes), "GB/s": probe_bytes / (probe_ms * 1e-3) / 1e9,
                 "kernel": "probe_gather_read_kernel (whole 4 KiB blocks, no arithmetic)"},
+            "bare_read_of_as_many_consecutive_blocks": {
+                "ms": run_ms, "bytes": int(probe_bytes), "GB/s": probe_bytes / (run_ms * 1e-3) / 1e9},
         },
     }
     if not args.no_cpu_baseline:
