@@ -332,6 +332,37 @@ def bench_cache_write(args):
             raise RuntimeError(f"mux_probe_scatter_copy returned {rc}")
 
     ms_scopy = _time(scatter, args.steps, args.warmup)
+    # Where the blocks lie matters for writes (it does not for reads): the same step and the same
+    # probe with the step's blocks (a) as runs of 52 consecutive ids - what a layer's slice of the
+    # allocator's [token block][layer][head] order looks like (csrc/memory_manager.cpp:104-135) -
+    # and (b) as one consecutive run of the pool.
+    by_pattern = {"random_permutation": {"kernel_ms": ms_p, "probe_ms": ms_scopy}}
+    n_tb = per_set // 52
+    for name, make in (("runs_of_52_consecutive_blocks",
+                        lambda: (rng.choice(N // 52 - 1, size=n_tb, replace=False)[:, None] * 52 + np.arange(52)).reshape(-1)),
+                       ("one_consecutive_run", lambda: np.arange(per_set) + int(rng.integers(0, N - per_set)))):
+        alt = []
+        for i in range(5):
+            slots, _ = workloads.prefill_slot_mapping(lens, 52, bs, make())
+            alt.append(torch.from_numpy(slots).to(dev))
+        alt_ids = [(ds[::bs, 0, :] // bs).reshape(-1).to(torch.int32).contiguous() for ds in alt]
+
+        def write_alt(i):
+            kv = psets[i % 5][0]
+            ops.reshape_and_cache(kv[:, :52 * D], kv[:, 52 * D:], k_pool, v_pool, alt[i % 5])
+
+        def scatter_alt(i):
+            f, ids = flat[i % 5], alt_ids[i % 5]
+            rc = _l.probe().mux_probe_scatter_copy(k_pool.data_ptr(), v_pool.data_ptr(), N, f.data_ptr(),
+                                                   f[n_blk * 2048:].data_ptr(), ids.data_ptr(), n_blk, st)
+            if rc != 0:
+                raise RuntimeError(f"mux_probe_scatter_copy returned {rc}")
+
+        by_pattern[name] = {"kernel_ms": _time(write_alt, args.steps, args.warmup),
+                            "probe_ms": _time(scatter_alt, args.steps, args.warmup)}
+    for v in by_pattern.values():
+        v["kernel_frac_of_hbm"] = bytes_p / (v["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+        v["probe_frac_of_hbm"] = 2 * half / (v["probe_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS
     for i in range(5):          # the pool holds the probe's bytes now: put the step's own back
         write(i)
     gbs = bytes_p / (ms_p * 1e-3) / 1e9
@@ -341,6 +372,7 @@ def bench_cache_write(args):
                                                  "torch_copy_ms": ms_tcopy, "torch_copy_gbs": 2 * half / (ms_tcopy * 1e-3) / 1e9,
                                                  "scattered_to_the_steps_pool_blocks_ms": ms_scopy,
                                                  "scattered_to_the_steps_pool_blocks_gbs": 2 * half / (ms_scopy * 1e-3) / 1e9},
+           "by_where_the_blocks_lie": by_pattern,
            "decode_shape": "7b/13b/30b, 56 tokens, three launches", "decode_ms": ms_d, "decode_bytes": bytes_d,
            "decode_gbs": bytes_d / (ms_d * 1e-3) / 1e9,
            "decode_one_fused_launch_ms": ms_d1, "decode_one_fused_launch_with_rope_ms": ms_dr,
