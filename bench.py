@@ -69,7 +69,7 @@ def parse():
                     help="prefill_timeline: 16 prompts of 2048 tokens, 32 heads, instead of the three-model mix")
     ap.add_argument("--workload", default="mixed3_decode",
                     choices=["mixed3_decode", "prefill3", "cache_write", "colocated", "gqa_long", "model_ops", "host_step",
-                             "cu_masks", "prefill_long", "decode_timeline", "prefill_timeline", "mfma_ceiling"],
+                             "cu_masks", "prefill_long", "decode_timeline", "prefill_timeline", "gqa_timeline", "mfma_ceiling"],
                     help="mixed3_decode is the headline metric; the others are the remaining synthetic "
                          "shapes, each printing its own JSON line")
     return ap.parse_args()
@@ -714,6 +714,69 @@ def bench_prefill_timeline(args):
                   "traffic": None, "kernel": "prefill_causal_kernel<F16> with workgroup stamps"}, higher=False)
 
 
+def bench_gqa_timeline(args):
+    """Residency of the workgroups of one launch of the grouped-query decode
+    kernel on the long-context workload, from the tracing build of the library
+    (entry and end stamps of every workgroup, 100 MHz clock)."""
+    import ctypes
+    import torch
+    from muxserve_amd import _lib, ops, workloads
+    from muxserve_amd.build import TRACE_LIB
+    from muxserve_amd.pool import allocate_gpu_cache
+    if os.path.abspath(_lib.ATTN_LIB_PATH) != os.path.abspath(TRACE_LIB):
+        raise SystemExit("gqa_timeline needs the tracing build: python -m muxserve_amd.build trace, then run with "
+                         f"MUXSERVE_ATTN_LIB={TRACE_LIB}")
+    lib = _lib.attn()
+    lib.mux_decode_trace_set.restype = ctypes.c_int32
+    lib.mux_decode_trace_set.argtypes = [ctypes.c_void_p, ctypes.c_int64]
+    dev, bs = "cuda:0", 16
+    N = int(200e9) // 8192 // 128 * 128
+    k_pool, v_pool = allocate_gpu_cache(N, bs, dev, dtype=torch.bfloat16)
+    sets = [workloads.config5(seed=args.seed + i, num_pool_blocks=N)[0][0].to_device(dev, torch.bfloat16, seed=i)
+            for i in range(3)]
+    launches = [ops.DecodeLaunch([ops.DecodeCall(m.out, m.q, m.d_block_tables, m.d_context_lens, m.max_context_len, m.scale,
+                                                 total_context_len=int(m.context_lens.sum()),
+                                                 context_lens_host=None if args.no_host_lens else torch.from_numpy(
+                                                     np.ascontiguousarray(m.context_lens, dtype=np.int32)))],
+                                 k_pool, v_pool, partition_size=args.partition) for m in sets]
+    rows = 16384
+    table = torch.zeros((rows, 8), dtype=torch.int64, device=dev)
+    for i in range(30):
+        launches[i % 3]()
+    torch.cuda.synchronize()
+    slots = 2 * torch.cuda.get_device_properties(0).multi_processor_count
+    per_batch = []
+    for which in range(3):
+        table.zero_()
+        launches[(which + 1) % 3]()                      # a launch right before, as in the benchmark loop
+        assert lib.mux_decode_trace_set(table.data_ptr(), rows) == 0
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        launches[which]()
+        e1.record()
+        torch.cuda.synchronize()
+        lib.mux_decode_trace_set(None, 0)
+        t = table.cpu().numpy()
+        t = t[(t[:, 6] > 0) & ((t[:, 7] & 0xffff) > 0)]      # workgroups that had a unit
+        base = t[:, 0].min()
+        a, g = (t[:, 0] - base) / 100.0, (t[:, 6] - base) / 100.0
+        ntok = t[:, 7] & 0xffff
+        span, life = float(g.max()), g - a
+        full = ntok >= 0.95 * ntok.max()
+        per_batch.append({"kernel_us_with_stamps": e0.elapsed_time(e1) * 1e3, "span_us": span, "workgroups": int(len(t)),
+                          "life_us_mean": float(life.mean()), "life_us_of_the_full_units": float(life[full].mean()),
+                          "tokens_of_a_full_unit": int(ntok.max()),
+                          "slot_time_filled": float(life.sum() / (span * slots)), "last_start_us": float(a.max()),
+                          "ends_us_p50_p90_max": [float(np.percentile(g, 50)), float(np.percentile(g, 90)), span],
+                          "resident_every_10us": [int(((a <= lo + 5) & (g > lo + 5)).sum())
+                                                  for lo in np.arange(0.0, span + 10.0, 10.0)]})
+    span = float(np.mean([b["span_us"] for b in per_batch]))
+    cfg = {"workload": "gqa_timeline", "partition": args.partition, "workgroup_slots": int(slots), "batches": per_batch}
+    return _line("grouped-query decode kernel workgroup residency (tracing build)", span, "us", args, span * 1e-3, cfg,
+                 {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": None, "traffic": None,
+                  "kernel": "paged_decode_gqa_kernel<BF16,16,8,4> with entry and end stamps"}, dtype="bf16", higher=False)
+
+
 def bench_gqa_long(args):
     """Config 5: 64 query heads over 8 kv heads, bf16, batch 64, ctx U[2048, 8192]."""
     import torch
@@ -990,7 +1053,7 @@ def main():
               file=sys.stderr)
         sys.exit(2)
     other = {"prefill3": bench_prefill3, "cache_write": bench_cache_write, "colocated": bench_colocated, "cu_masks": bench_cu_masks, "prefill_long": bench_prefill_long, "decode_timeline": bench_decode_timeline,
-             "prefill_timeline": bench_prefill_timeline,
+             "prefill_timeline": bench_prefill_timeline, "gqa_timeline": bench_gqa_timeline,
              "gqa_long": bench_gqa_long, "model_ops": bench_model_ops, "host_step": bench_host_step,
              "mfma_ceiling": bench_mfma_ceiling}
     if args.workload in other:

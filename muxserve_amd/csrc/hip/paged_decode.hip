@@ -47,6 +47,7 @@ thread_local int32_t g_last_hip_error = 0;
 // workgroup: [0] entry, [1] unit known, [2] block ids and q there, [3] K/V loads
 // of the (last) tile issued, [4] tile consumed, [5] past the workgroup's barrier,
 // [6] merge / publish / combine done, [7] tokens of the unit | split << 16.
+// The matrix-core kernel of the grouped-query shapes stamps [0], [6] and [7] only.
 #ifdef MUX_TRACE
 __device__ long long *g_decode_trace = nullptr;
 __device__ long long g_decode_trace_rows = 0;
@@ -1157,6 +1158,7 @@ __device__ __forceinline__ bool decode_unit_gqa(const DecodeParams &P, const Dec
 
 template <typename T, int BS, int G, int NW>
 __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const DecodeParams P) {
+  MUX_TR(0);
   __shared__ GqaSmem<T, G, NW> sm;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1172,7 +1174,13 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
   Unit u;
   u.item = ii;
   u.wh = local - e * WH;
+#ifdef MUX_TRACE
+  u.t0 = u.t1 = 0, u.n_splits = 0;       // (a workgroup that finds no unit reports no tokens)
+#endif
   decode_unit_gqa<T, BS, G, NW, false>(P, I, u, e, sm, lane, wave);
+  // (tracing build: the matrix-core kernel stamps its entry and its end only)
+  MUX_TR(6);
+  MUX_TRV(7, static_cast<long long>(u.t1 - u.t0) | (static_cast<long long>(u.n_splits > 1) << 16));
 }
 
 // (pairs that got no place in the grid: see paged_decode_sweep_kernel)
