@@ -36,9 +36,9 @@ MFMA_PEAK_TFLOPS = 2500.0     # dense fp16 / bf16
 # profiles/paged_decode_mixed3_hbm_traffic.txt (420.6 MB measured / 410.6 MB).
 MIXED3_TRAFFIC_RATIO = 1.024
 # Same for the grouped-query decode kernel (profiles/paged_decode_gqa_long_kernel_trace_and_traffic.txt:
-# 1390.0 MB / 1358.8 MB) and the prefill-shaped cache write
+# 1369.5 MB / 1358.8 MB) and the prefill-shaped cache write
 # (profiles/reshape_and_cache_write_kernel_trace_and_traffic.txt: 231.9 MB / 219.8 MB).
-GQA_LONG_TRAFFIC_RATIO = 1.023
+GQA_LONG_TRAFFIC_RATIO = 1.008
 CACHE_WRITE_TRAFFIC_RATIO = 1.055
 
 
@@ -744,7 +744,7 @@ def bench_gqa_timeline(args):
     for i in range(30):
         launches[i % 3]()
     torch.cuda.synchronize()
-    slots = 2 * torch.cuda.get_device_properties(0).multi_processor_count
+    slots = 3 * torch.cuda.get_device_properties(0).multi_processor_count       # 142 registers: three workgroups per CU
     per_batch = []
     for which in range(3):
         table.zero_()

@@ -114,7 +114,9 @@ int32_t mux_reshape_and_cache(const void *k, const void *v, int64_t kv_row_strid
  * partition_size: tokens per split of a context (multiple of 64), 0 = choose:
  * 256, or 1024 for a large launch (at least 1.5 M tokens x head groups over
  * its models, by total_context_len or by num_seqs * max_context_len / 2 without
- * it), or 512 / 1024 when contexts exceed 4096 tokens.  The workspace size
+ * it), or 512 when contexts exceed 4096 tokens; when every model of the launch
+ * has four or more query heads per kv head: that sum / 768 (a workgroup slot's
+ * share of the launch), rounded up to a multiple of 256.  The workspace size
  * reported for 0 covers every choice, so it may differ from launch to launch.
  * workspace: scratch for the partial results of split contexts and, for
  * batches of more than 256 sequences, the table that maps workgroups to

@@ -880,8 +880,8 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_sweep_kernel(const Decod
 // so every K and V load lands in its operand register straight from the pool.
 // The score accumulators give a lane tokens 16 tg + 4 g + i of its head; the
 // regrouping into runs of 8 tokens goes through 1 KiB of LDS per wave.
-// A wave advances 32 tokens per step with two register sets, so the loads of
-// the next step are in flight while the current one is consumed.
+// A wave advances 32 tokens per step (16 KiB of K/V in 64 registers); three
+// waves per SIMD keep the memory system busy while one of them computes.
 // Work units, partitions, the cross-wave merge and the split combine are those
 // of the kernel above.
 // ---------------------------------------------------------------------------
@@ -1105,35 +1105,25 @@ __device__ __forceinline__ bool decode_unit_gqa(const DecodeParams &P, const Dec
     }
   };
 
-  // Two register sets: the loads of the next step are in flight while the
-  // current one is consumed.  Vector loads return in order, so waiting for a
-  // step's block ids also waits for every load issued before them: the ids of
-  // step s + 2 are therefore requested BEFORE the K/V loads of step s + 1 go
-  // out (two id registers in rotation), and waiting for them never waits for
-  // K/V that is still wanted in flight.
+  // One register set per wave and three waves per SIMD: while a wave consumes
+  // its step the SIMD's other two have theirs in flight (two sets and two waves
+  // per SIMD moved as much on long launches and less on short ones: 76 against
+  // 67 us on 16 contexts of 2048-8192 tokens, 46 against 37 us on 64 contexts of
+  // 256-1024).  Vector loads return in order, so waiting for a step's block ids
+  // also waits for every load issued before them: the ids of step s + 1 are
+  // therefore requested BEFORE the K/V loads of step s go out, and waiting for
+  // them never waits for K/V that is still wanted in flight.
   int tb = u.t0 + kGqaTile * wave;
   if (tb < t1) {
-    GqaTile ra, rb;
-    int3 ids_a = load_ids(tb);
-    int3 ids_b = make_int3(0, 0, 0);
-    if (tb + kStep < t1) ids_b = load_ids(tb + kStep);
-    issue(ra, tb, ids_a);
+    GqaTile r;
+    int3 ids_next = load_ids(tb);
     while (true) {
-      const bool has_b = tb + kStep < t1;
-      if (has_b) {
-        if (tb + 2 * kStep < t1) ids_a = load_ids(tb + 2 * kStep);
-        issue(rb, tb + kStep, ids_b);
-      }
-      compute(ra, tb);
-      if (!has_b) break;
-      tb += kStep;
-      const bool has_a = tb + kStep < t1;
-      if (has_a) {
-        if (tb + 2 * kStep < t1) ids_b = load_ids(tb + 2 * kStep);
-        issue(ra, tb + kStep, ids_a);
-      }
-      compute(rb, tb);
-      if (!has_a) break;
+      const int3 ids = ids_next;
+      const bool more = tb + kStep < t1;
+      if (more) ids_next = load_ids(tb + kStep);
+      issue(r, tb, ids);
+      compute(r, tb);
+      if (!more) break;
       tb += kStep;
     }
   }
@@ -1157,7 +1147,7 @@ __device__ __forceinline__ bool decode_unit_gqa(const DecodeParams &P, const Dec
 }
 
 template <typename T, int BS, int G, int NW>
-__global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const DecodeParams P) {
+__global__ __launch_bounds__(64 * NW, 3) void paged_decode_gqa_kernel(const DecodeParams P) {
   MUX_TR(0);
   __shared__ GqaSmem<T, G, NW> sm;
   const int lane = threadIdx.x & 63;
@@ -1185,7 +1175,7 @@ __global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_kernel(const Deco
 
 // (pairs that got no place in the grid: see paged_decode_sweep_kernel)
 template <typename T, int BS, int G, int NW>
-__global__ __launch_bounds__(64 * NW, 2) void paged_decode_gqa_sweep_kernel(const DecodeParams P) {
+__global__ __launch_bounds__(64 * NW, 3) void paged_decode_gqa_sweep_kernel(const DecodeParams P) {
   __shared__ GqaSmem<T, G, NW> sm;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1220,8 +1210,7 @@ int pick_group(int ratio);
 
 // Tokens per partition when the caller leaves the choice to the library: short
 // partitions spread the batch over more workgroups, long ones amortise a unit's
-// fixed cost; the grouped-query kernel streams a partition with its loads
-// overlapped and prefers the longer ones.
+// fixed cost and split fewer contexts.
 int choose_partition(const MuxDecodeItem *items, int n_items, int requested) {
   if (requested > 0) return requested;
   int max_ctx = 0;
@@ -1240,12 +1229,24 @@ int choose_partition(const MuxDecodeItem *items, int n_items, int requested) {
                                : static_cast<int64_t>(it.num_seqs) * (it.max_context_len / 2);
     token_heads += tokens * (it.num_q_heads / std::max(group, 1));
   }
-  if (max_ctx > 4096) return all_grouped ? 1024 : 512;
+  // Grouped-query launches: as many tokens per unit as a workgroup slot's share
+  // of the launch (three workgroups on each of the 256 compute units), so that
+  // the units fill the chip about once and few contexts are split at all; never
+  // under 256.  Against the 1024 / 256 tokens used before: 230 against 237 us on
+  // 64 contexts of 2048-8192 tokens, 245 against 315 us on 512 of 256-1024, 19.5
+  // against 26 us on two long ones (their units now fill a fifth of the chip
+  // instead of a twentieth).
+  if (all_grouped) {
+    constexpr int64_t kSlots = 3 * 256;
+    const int64_t per_slot = (token_heads / kSlots + 255) / 256 * 256;
+    return static_cast<int>(std::min<int64_t>(std::max<int64_t>(per_slot, 256), 1 << 20));
+  }
+  if (max_ctx > 4096) return 512;
   // A large launch does better with long partitions (fewer units, hardly any
   // hand-off: 1 - 6 % over launches of 0.8 - 1.7 GB of K/V, one model or three);
   // a small one needs the many short units to fill the chip and to end evenly
   // (1024-token partitions: +1 to +15 % there).
-  if (!all_grouped && token_heads >= 1500000) return 1024;
+  if (token_heads >= 1500000) return 1024;
   return 256;
 }
 

@@ -135,7 +135,8 @@ def test_library_chosen_partition_follows_the_size_of_the_launch():
     """With partition_size 0 the library picks the partition: 256 tokens, but
     1024 for a large launch (at least 1.5 M tokens x heads over its models, by
     the caller's bound on the context sum, or by half the longest context per
-    sequence without one) and 512 beyond 4096-token contexts.  Seen through the
+    sequence without one) and 512 beyond 4096-token contexts; for launches of
+    grouped-query models only, a workgroup slot's share of the launch.  Seen through the
     unit count of the host-side enumeration; the workspace asked for is never
     smaller than what the 256-token partition needs, whichever is picked."""
     import numpy as np
@@ -184,6 +185,26 @@ def test_library_chosen_partition_follows_the_size_of_the_launch():
     # contexts beyond 4096 tokens: 512-token partitions for the vector-ALU kernel
     it, ctx = item(4, 32, 5000, 4 * 5000)
     assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, 0) == units(ctx, 512)
+
+    # Grouped-query launches (8 query heads per kv head): a workgroup slot's share of the launch -
+    # tokens x kv heads / (3 x 256 slots), rounded up to 256 tokens, never under 256.
+    def gqa_item(B, ctx_value, hint):
+        it, ctx = item(B, 64, ctx_value, hint)
+        it.num_kv_heads = 8
+        return it, ctx
+
+    it, ctx = gqa_item(64, 5120, 64 * 5120)          # 64 x 5120 x 8 / 768 = 3413 -> 3584 tokens
+    assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, 0) == units(ctx, 3584) == 2 * 64
+    it, ctx = gqa_item(16, 5120, 16 * 5120)          # 853 -> 1024
+    assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, 0) == units(ctx, 1024) == 5 * 16
+    it, ctx = gqa_item(2, 5120, 2 * 5120)            # 107 -> 256: a small launch is spread over many units
+    assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, 0) == units(ctx, 256) == 20 * 2
+    it, ctx = gqa_item(256, 1000, 256 * 1000)        # 2667 -> 2816: beyond every context, nothing is split
+    assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, 0) == 256
+    big = lib.mux_paged_decode_workspace_bytes(ctypes.addressof(it), 1, 0)
+    assert big == lib.mux_paged_decode_workspace_bytes(ctypes.addressof(it), 1, 256)
+    it, ctx = gqa_item(64, 5120, 0)                  # no bound: half the longest context each, 1707 -> 1792
+    assert lib.mux_paged_decode_host_pairs(ctypes.addressof(it), 1, 0) == units(ctx, 1792) == 3 * 64
 
 
 # ---------------------------------------------------------------------------
