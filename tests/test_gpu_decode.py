@@ -534,6 +534,33 @@ def test_decode_large_single_model_batch_takes_the_long_partitions(host_lens):
     assert (got - short).abs().max().item() <= 1e-3
 
 
+@pytest.mark.parametrize("shape", ["a slot's share splits the long contexts", "a slot's share beyond every context",
+                                   "two long contexts in many short units"])
+def test_decode_grouped_query_launch_takes_a_slots_share_as_partition(shape):
+    """Launches of grouped-query models only: with partition_size 0 the library
+    takes tokens x kv heads / 768 workgroup slots, rounded up to 256 tokens, as
+    partition.  Against the oracle, host- and device-enumerated (the same units:
+    the same bits), and against the same batch in 256-token partitions."""
+    _announce(f"grouped-query partition policy: {shape}")
+    rng = np.random.Generator(np.random.PCG64(91))
+    if shape.startswith("a slot's share splits"):
+        ctx = rng.integers(150, 1301, size=96).astype(np.int32)      # 96 x ~725 x 8 / 768 -> 768-token partitions
+        ctx[:4] = (768, 784, 785, 1300)
+        hq, hkv = 32, 8
+    elif shape.startswith("a slot's share beyond"):
+        ctx = rng.integers(100, 701, size=300).astype(np.int32)      # 300 x ~400 x 8 / 768 -> 1280: nothing is split
+        hq, hkv = 64, 8
+    else:
+        ctx = np.asarray([2500, 3100], dtype=np.int32)               # 5600 x 8 / 768 -> 256-token partitions
+        hq, hkv = 64, 8
+    got, want = _decode_case(92, ctx, hq, hkv, 16, hint=True, host_lens=True)
+    _check(got, want)
+    dev_enum, _ = _decode_case(92, ctx, hq, hkv, 16, hint=True, host_lens=False)
+    assert torch.equal(got, dev_enum)
+    short, _ = _decode_case(92, ctx, hq, hkv, 16, partition=256, hint=True, host_lens=True)
+    assert (got - short).abs().max().item() <= 1e-3
+
+
 def test_decode_rejects_bad_arguments():
     _announce("decode argument validation")
     dk, dv = allocate_gpu_cache(8, 16, DEV)
