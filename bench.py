@@ -425,7 +425,7 @@ def bench_colocated(args):
     def prefill(i, stream=None):
         ops.prefill_causal(pout, q, k, v, cu, 1024, D ** -0.5, 52, stream=stream)
 
-    steps, warm = args.steps, args.warmup
+    steps, warm = args.steps, max(args.warmup, PREFILL_MIN_WARMUP)      # (the prefill's clock: see PREFILL_MIN_WARMUP)
     res = {"decode_alone_full_ms": _time(decode, steps, warm), "prefill_alone_full_ms": _time(prefill, steps, warm)}
     res["decode_alone_60pct_ms"] = _time(lambda i: decode(i, s_dec), steps, warm, s_dec.torch_stream)
     res["prefill_alone_40pct_ms"] = _time(lambda i: prefill(i, s_pre), steps, warm, s_pre.torch_stream)
